@@ -609,8 +609,16 @@ class WindowAttentionSpec:
     ``sink`` adds one to the softmax denominator (a key of score 0 without a value),
     ``gate`` multiplies head h's output by sigmoid of a per-head projection of the mixer input,
     ``bias`` adds biases in the q / k / v projections, ``qk_norm`` applies a weighted RMS norm
-    over the WHOLE q (and k) projection before the rotation, ``v_norm`` divides every value
-    head by its root mean square (cached so)."""
+    over the WHOLE q (and k) projection before the rotation, ``head_norm`` one over every
+    query / key head with a weight of ``dim`` elements that all heads share, ``v_norm`` divides
+    every value head by its root mean square (cached so), ``out_bias`` adds a bias in the
+    output projection.
+
+    ``maps`` = 2 is differential attention: every query head and every key head carries two
+    maps side by side ([map 1 | map 2], ``dim`` each); each map is a softmax attention of its
+    own over the same values, and the head's output is ``a1 - lam * a2`` divided by its root
+    mean square, times ``1 - diff`` (``lam`` comes from learned vectors and ``diff``).
+    ``kv_from`` = j: the layer has no key / value projections and reads layer j's cache."""
     heads: int
     kv_heads: int
     dim: int            # query / key dims per head
@@ -624,16 +632,21 @@ class WindowAttentionSpec:
     bias: bool = False
     qk_norm: bool = False
     v_norm: bool = False
+    head_norm: bool = False
+    out_bias: bool = False
+    maps: int = 1
+    diff: float = 0.0
+    kv_from: int | None = None
 
     kind = "attention"
 
     @property
     def q_size(self) -> int:
-        return self.heads * self.dim
+        return self.heads * self.maps * self.dim
 
     @property
     def k_size(self) -> int:
-        return self.kv_heads * self.dim
+        return self.kv_heads * self.maps * self.dim
 
     @property
     def v_size(self) -> int:
@@ -641,8 +654,26 @@ class WindowAttentionSpec:
 
     @property
     def cache_dim(self) -> int:
-        """Cached elements per token: all key heads, then all value heads."""
-        return self.k_size + self.v_size
+        """Cached elements per token: all key heads, then all value heads (none when the layer
+        reads another layer's cache)."""
+        return 0 if self.kv_from is not None else self.k_size + self.v_size
+
+
+@dataclass(frozen=True)
+class WkvSpec:
+    """Linear attention with a decay per key channel and token (RWKV-style time mixing): every
+    projection reads its own blend of the token's and the previous token's input, the decay
+    comes from a ``decay_rank`` bottleneck, the current token enters its own read-out through a
+    bonus vector, and the per-head ``dim x dim`` state is 32-bit."""
+    heads: int
+    dim: int
+    decay_rank: int = 0     # read from the checkpoint when 0
+
+    kind = "wkv"
+
+    @property
+    def size(self) -> int:
+        return self.heads * self.dim
 
 
 @dataclass(frozen=True)
@@ -697,11 +728,28 @@ class ParallelMixerSpec:
 
 @dataclass(frozen=True)
 class DenseFFSpec:
-    """down(act(up(x))) with one of the op set's elementwise activations."""
+    """down(act(up(x))) with one of the op set's elementwise activations (``xielu``, ``relu2``)."""
     ff: int
     act: str = "xielu"
 
     kind = "dense"
+
+
+@dataclass(frozen=True)
+class RoutedMoESpec:
+    """Mixture of gated feed-forwards with a learned softmax router: the ``top`` experts with
+    the largest score + correction are chosen, weighted by their (uncorrected, not
+    renormalised) score times ``scale``. The last ``identity`` router outputs are experts
+    without weights that return their input; ``shared_ff`` > 0 adds a gated feed-forward that
+    every token runs."""
+    experts: int
+    top: int
+    ff: int
+    identity: int = 0
+    scale: float = 1.0
+    shared_ff: int = 0
+
+    kind = "routed_moe"
 
 
 @dataclass(frozen=True)
@@ -899,6 +947,104 @@ class FikizenConfig:
             bos_token_id=d.get("bos_token_id"), eos_token_id=eos)
 
 
+@dataclass(frozen=True)
+class KemavikConfig:
+    """Kemavik: a decoder given as a list of layers whose norms sit on the sublayers' OUTPUTS
+    (``x <- x + norm(mixer(x))``, ``x <- x + norm(ff(x))``, one-plus-weight RMS norms). Mixers:
+    RWKV-style linear attention with per-channel decays, or differential grouped-query
+    attention with per-head query / key norms (a layer may read another layer's keys and
+    values). Feed-forwards: dense with a squared ReLU, or a routed mixture of gated experts
+    with identity experts and a shared expert."""
+    name: str = "kemavik"
+    architecture: str = "kemavik"
+    family: str = "kemavik"
+    hidden_size: int = 256
+    vocab_size: int = 512
+    layers: tuple = ()
+    norm_eps: float = 1e-6
+    max_position_embeddings: int = 1 << 20   # no position tables
+    default_model_len: int = 32768
+    bos_token_id: int | None = None
+    eos_token_id: tuple = ()
+    vision: object = None
+    num_experts: int = 0                      # engine start-up tuning of the dense families keys on it
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def runs(self) -> list:
+        """Layer runs in execution order: (layer index, 0, False); every layer runs once."""
+        return [(i, 0, False) for i in range(len(self.layers))]
+
+    def num_params(self) -> int:
+        H, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size
+        for l in self.layers:
+            m, f = l.mixer, l.mlp
+            if isinstance(m, WkvSpec):
+                n += 5 * H * m.size + 2 * (m.decay_rank or 64) * H
+            else:
+                n += H * (m.q_size + m.cache_dim) + m.heads * m.vdim * H
+            if isinstance(f, DenseFFSpec):
+                n += 2 * f.ff * H
+            elif f is not None:
+                n += 3 * H * (f.experts * f.ff + f.shared_ff) + H * (f.experts + f.identity)
+        return n
+
+    def replace(self, **kw) -> "KemavikConfig":
+        return dataclasses.replace(self, **kw)
+
+    @staticmethod
+    def from_dict(d: dict, name: str = "model") -> "KemavikConfig":
+        layers = []
+        for i, l in enumerate(d["layers"]):
+            m, kind = l["mixer"], l["type"]
+            if kind == "wkv":
+                mixer = WkvSpec(heads=int(m["heads"]), dim=int(m["dim"]), decay_rank=int(m.get("decay_rank") or 0))
+            elif kind == "attention":
+                src = m.get("kv_from")
+                mixer = WindowAttentionSpec(
+                    heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                    scale=float(m["scale"]), bias=True, out_bias=True, head_norm=True, maps=2,
+                    diff=float(m["diff"]), kv_from=None if src is None else int(src))
+            else:
+                raise NotImplementedError(f"unknown mixer {kind!r}")
+            f = l.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind") == "dense":
+                    mlp = DenseFFSpec(ff=int(f["ff"]), act="relu2")
+                elif f.get("kind") == "moe":
+                    r = f["router"]
+                    mlp = RoutedMoESpec(experts=int(r["experts"]), top=int(r["top"]), ff=int(f["expert"]["ff"]),
+                                        identity=int(r.get("identity") or 0), scale=float(r.get("scale", 1.0)),
+                                        shared_ff=int((f.get("shared") or {}).get("ff") or 0))
+                else:
+                    raise NotImplementedError(f"unknown feed-forward {f.get('kind')!r}")
+            layers.append(HybridLayerSpec(mixer, mlp))
+        check_kv_sources(layers)
+        norm = d.get("norm") or {}
+        eos = d.get("eos_token_id", ())
+        eos = tuple(eos) if isinstance(eos, (list, tuple)) else (eos,)
+        return KemavikConfig(
+            name=name, hidden_size=int(d["width"]), vocab_size=int(d["vocab"]), layers=tuple(layers),
+            norm_eps=float(norm.get("eps", 1e-6)), bos_token_id=d.get("bos_token_id"), eos_token_id=eos)
+
+
+def check_kv_sources(layers):
+    """A layer that reads another layer's keys and values must name an earlier attention layer
+    with a cache of its own and the same key / value head layout."""
+    for i, l in enumerate(layers):
+        j = getattr(l.mixer, "kv_from", None)
+        if j is None:
+            continue
+        if not (0 <= j < i) or not isinstance(layers[j].mixer, WindowAttentionSpec) or layers[j].mixer.kv_from is not None:
+            raise ValueError(f"layer {i}: kv_from must name an earlier attention layer with keys and values of its own")
+        a, b = l.mixer, layers[j].mixer
+        if (a.kv_heads, a.maps, a.dim, a.vdim) != (b.kv_heads, b.maps, b.dim, b.vdim):
+            raise ValueError(f"layer {i}: its key / value heads differ from those of layer {j}, whose cache it reads")
+
+
 def config_from_dict(d: dict, name: str = "model"):
     """Model config of a ``config.json``: the layer-list designs are recognised by their
     ``architecture`` key, everything else is a HuggingFace config."""
@@ -907,6 +1053,8 @@ def config_from_dict(d: dict, name: str = "model"):
         return HybridConfig.from_dict(d, name=name)
     if arch == "fikizen":
         return FikizenConfig.from_dict(d, name=name)
+    if arch == "kemavik":
+        return KemavikConfig.from_dict(d, name=name)
     return ModelConfig.from_hf_dict(d, name=name)
 
 
@@ -962,4 +1110,32 @@ PRESETS.update({
                                    dict(heads=8, kv_heads=4, dim=64, vdim=64, scale=0.125, window=80, rot_dims=64),
                                    dict(heads=8, kv_heads=4, dim=64, vdim=64, conv=3), dict(heads=8, dim=64, decay_rank=32),
                                    1536, "adAp"),
+})
+
+
+def _mini_kemavik(name, H, V, wkv, attn, ff, moe, order):
+    """order: 'w' linear attention + dense feed-forward, 'a' differential attention + routed experts,
+    's' differential attention on the keys and values of the nearest 'a' before it + dense feed-forward,
+    'n' linear attention without a feed-forward."""
+    layers = []
+    for c in order:
+        if c in "wn":
+            layers.append(HybridLayerSpec(WkvSpec(**wkv), DenseFFSpec(ff, "relu2") if c == "w" else None))
+        else:
+            src = max(i for i, o in enumerate(order[:len(layers)]) if o == "a") if c == "s" else None
+            a = WindowAttentionSpec(bias=True, out_bias=True, head_norm=True, maps=2, kv_from=src, **attn)
+            layers.append(HybridLayerSpec(a, RoutedMoESpec(**moe) if c == "a" else DenseFFSpec(ff, "relu2")))
+    return KemavikConfig(name=name, hidden_size=H, vocab_size=V, layers=tuple(layers), eos_token_id=(2,),
+                         bos_token_id=1)
+
+
+PRESETS.update({
+    # CPU plumbing size
+    "tiny-kemavik": _mini_kemavik("tiny-kemavik", 64, 320, dict(heads=2, dim=16, decay_rank=8),
+                                  dict(heads=4, kv_heads=2, dim=8, vdim=24, scale=0.3, diff=0.4), 96,
+                                  dict(experts=5, top=2, ff=24, identity=2, scale=1.5, shared_ff=40), "wasaw"),
+    # GPU-test size
+    "small-kemavik": _mini_kemavik("small-kemavik", 512, 1024, dict(heads=8, dim=64, decay_rank=32),
+                                   dict(heads=8, kv_heads=2, dim=32, vdim=64, scale=32 ** -0.5, diff=0.5), 1536,
+                                   dict(experts=8, top=2, ff=256, identity=2, scale=1.0, shared_ff=512), "wasw"),
 })

@@ -20,9 +20,19 @@ them is one op of the op set:
   ``expert_gemm`` launches (squared-ReLU in the first one's epilogue); the weighted
   combine is folded into the residual update (``scaled_add_group_rmsnorm``).
 * window attention: merged [q | k | v | gate] projection (biases in its epilogue) ->
-  ``attn_prepare`` (whole-projection q / k norm, rotation, value norm, paged cache write) ->
-  ``window_attention`` (sliding window, softmax with a sink, per-head output gate) ->
-  output projection.
+  ``attn_prepare`` (whole-projection or per-head q / k norm, rotation, value norm, paged cache
+  write) -> ``window_attention`` (sliding window, softmax with a sink, per-head output gate; with
+  two maps per head the differential combination and its norm) -> output projection. A layer
+  that reads another layer's cache projects only its queries.
+* linear attention with per-channel decays (``Wkv``): ``token_shift`` (five blends of the token's
+  and the previous token's 32-bit input) -> one batched projection for r / k / v / gate and the
+  decay bottleneck -> tanh -> decay up-projection (32-bit result) -> ``wkv`` (decay, bonus, the
+  recurrence from the sequence's state slot, per-head output norm and SiLU gate) -> output
+  projection.
+* routed experts (``RoutedMoE``): 32-bit router logits -> ``route_topk`` (softmax, corrected
+  selection, weights) -> ``moe_align`` tiles -> ``expert_gemm`` (gate | up) -> ``activation``
+  (silu_mul) -> ``expert_gemm`` (down); the weighted combine, the identity experts and the shared
+  expert are folded into the residual update (``add_normed``).
 * gated delta rule: merged [q | k | v | beta | decay | gate] projection -> ``gated_delta``
   (causal convolution + SiLU, unit q / k, the recurrence from the sequence's state slot,
   per-head output norm and SiLU gate) -> output projection.
@@ -42,7 +52,7 @@ import torch
 import torch.nn.functional as F
 
 from ..config import (DeltaRuleSpec, DenseFFSpec, GatedDeltaSpec, LatentAttentionSpec, MinGRUSpec, ParallelMixerSpec,
-                      TableMoESpec, WindowAttentionSpec)
+                      RoutedMoESpec, TableMoESpec, WindowAttentionSpec, WkvSpec)
 
 MOE_TILE = 32        # slots per expert tile of the expert GEMMs ...
 MOE_TILE_LARGE = 64  # ... when every expert has several tiles' worth of rows on average
@@ -262,44 +272,65 @@ class WindowAttention:
 
     def __init__(self, spec: WindowAttentionSpec, hidden: int, eps: float, device, dtype, ops):
         self.spec, self.hidden, self.eps, self.device, self.dtype, self.ops = spec, hidden, eps, device, dtype, ops
-        self.w_in = None     # [q | k | v | gate, hidden]
+        self.w_in = None     # [q | k | v | gate, hidden] (q alone when the layer reads another layer's cache)
         self.b_in = None     # [same] or None
-        self.q_norm = self.k_norm = None   # fp32 [heads * dim], [kv_heads * dim]
+        self.q_norm = self.k_norm = None   # fp32 [heads * dim], [kv_heads * dim]; [dim] each with head_norm
         self.w_o = None      # [hidden, heads * vdim]
+        self.b_o = None
+        self.lam = 0.0       # differential attention: weight of the second map
         half = spec.rot_dims // 2
         i = torch.arange(half, dtype=torch.float32)
         # f_i = base^(-2i / dims), 32-bit
         self.inv_freq = torch.pow(torch.tensor(spec.rot_base, dtype=torch.float32),
                                   -2.0 * i / max(spec.rot_dims, 1)).to(device)
         self.gate_off = spec.q_size + spec.cache_dim if spec.gate else -1
+        assert spec.maps in (1, 2) and not (spec.gate and spec.kv_from is not None)
 
     @property
     def out_size(self) -> int:
         return self.spec.heads * self.spec.vdim
 
+    def _in_names(self):
+        return ["q"] + (["k", "v"] if self.spec.kv_from is None else [])
+
     def load(self, get, prefix: str):
         s, dt, dev = self.spec, self.dtype, self.device
-        names = ["q", "k", "v"] + (["g"] if s.gate else [])
-        self.w_in = torch.cat([get(prefix + n) for n in names], 0).to(dev, dt).contiguous()
+        names = self._in_names()
+        self.w_in = torch.cat([get(prefix + n) for n in names + (["g"] if s.gate else [])], 0).to(dev, dt).contiguous()
         if s.bias:
-            b = [get(prefix + n + ".b") for n in ("q", "k", "v")] + ([torch.zeros(s.heads)] if s.gate else [])
+            b = [get(prefix + n + ".b") for n in names] + ([torch.zeros(s.heads)] if s.gate else [])
             self.b_in = torch.cat([x.float() for x in b]).to(dev, dt).contiguous()
-        if s.qk_norm:
+        if s.qk_norm or s.head_norm:
             self.q_norm = get(prefix + "q.norm").to(dev, torch.float32)
-            self.k_norm = get(prefix + "k.norm").to(dev, torch.float32)
+            if s.kv_from is None:
+                self.k_norm = get(prefix + "k.norm").to(dev, torch.float32)
+        if s.maps == 2:
+            # lam = exp(lq1 . lk1) - exp(lq2 . lk2) + diff, one number for the layer (32-bit)
+            lq1, lk1, lq2, lk2 = (get(prefix + n).to(torch.float32) for n in ("lq1", "lk1", "lq2", "lk2"))
+            self.lam = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum()) + torch.tensor(s.diff))
         self.w_o = get(prefix + "o").to(dev, dt).contiguous()
+        if s.out_bias:
+            self.b_o = get(prefix + "o.b").to(dev, dt).contiguous()
 
     def init_random(self, gen, std: float):
         s, H = self.spec, self.hidden
-        t = {"q": _rand(gen, s.q_size, H, std=std * 4), "k": _rand(gen, s.k_size, H, std=std * 4),
-             "v": _rand(gen, s.v_size, H, std=std * 4), "o": _rand(gen, H, self.out_size, std=std)}
+        t = {"q": _rand(gen, s.q_size, H, std=std * 4), "o": _rand(gen, H, self.out_size, std=std)}
+        if s.kv_from is None:
+            t.update({"k": _rand(gen, s.k_size, H, std=std * 4), "v": _rand(gen, s.v_size, H, std=std * 4)})
         if s.gate:
             t["g"] = _rand(gen, s.heads, H, std=std * 4)
         if s.bias:
-            t.update({"q.b": _rand(gen, s.q_size, std=0.3), "k.b": _rand(gen, s.k_size, std=0.3),
-                      "v.b": _rand(gen, s.v_size, std=0.3)})
+            t.update({n + ".b": _rand(gen, t[n].shape[0], std=0.3) for n in self._in_names()})
+        if s.out_bias:
+            t["o.b"] = _rand(gen, H, std=0.3)
         if s.qk_norm:
             t.update({"q.norm": 1.0 + 0.2 * _rand(gen, s.q_size), "k.norm": 1.0 + 0.2 * _rand(gen, s.k_size)})
+        if s.head_norm:
+            t.update({"q.norm": 1.0 + 0.2 * _rand(gen, s.dim), "k.norm": 1.0 + 0.2 * _rand(gen, s.dim)})
+        if (s.qk_norm or s.head_norm) and s.kv_from is not None:
+            del t["k.norm"]
+        if s.maps == 2:
+            t.update({n: _rand(gen, s.dim, std=0.2) for n in ("lq1", "lk1", "lq2", "lk2")})
         return t
 
     def mix(self, h, meta, cache, state, out, out_scale: float = 1.0):
@@ -308,12 +339,69 @@ class WindowAttention:
         s, ops = self.spec, self.ops
         proj = F.linear(h, self.w_in, self.b_in)
         ops.attn_prepare(proj, cache, meta, self.inv_freq, s, self.q_norm, self.k_norm, self.eps)
-        ops.window_attention(out, proj, cache, meta, s, self.gate_off, out_scale)
+        ops.window_attention(out, proj, cache, meta, s, self.gate_off, out_scale, self.lam, self.eps)
         return out
 
     def forward(self, h, meta, cache, state):
         out = torch.empty(h.shape[0], self.out_size, device=h.device, dtype=h.dtype)
-        return F.linear(self.mix(h, meta, cache, state, out), self.w_o)
+        return F.linear(self.mix(h, meta, cache, state, out), self.w_o, self.b_o)
+
+
+class Wkv:
+    cache_dim = 0
+    input32 = True      # forward reads the 32-bit stream itself, not its rounding to the activation type
+    BLENDS = ("r", "k", "v", "g", "w")
+
+    def __init__(self, spec: WkvSpec, hidden: int, eps: float, device, dtype, ops):
+        self.spec, self.hidden, self.eps, self.device, self.dtype, self.ops = spec, hidden, eps, device, dtype, ops
+        self.mu = None      # fp32 [5, hidden]: blend weights of r, k, v, gate, decay
+        self.w_in_t = None  # [4, hidden, heads * dim]: r, k, v, gate (transposed for the batched product)
+        self.w1 = None      # [rank, hidden]
+        self.w2 = None      # [heads * dim, rank]
+        self.w0 = self.u = self.norm = None   # fp32 [heads * dim]
+        self.w_o = None
+
+    @property
+    def out_size(self) -> int:
+        return self.spec.size
+
+    def state_shapes(self, slots: int):
+        s = self.spec
+        return [(slots, s.heads, s.dim, s.dim), (slots, self.hidden)]
+
+    def load(self, get, prefix: str):
+        dt, dev = self.dtype, self.device
+        self.mu = torch.stack([get(prefix + "mu." + n).float() for n in self.BLENDS]).to(dev).contiguous()
+        self.w_in_t = torch.stack([get(prefix + n) for n in ("r", "k", "v", "g")]).to(dev, dt).transpose(1, 2).contiguous()
+        self.w1 = get(prefix + "w1").to(dev, dt).contiguous()
+        self.w2 = get(prefix + "w2").to(dev, dt).contiguous()
+        self.w0 = get(prefix + "w0").to(dev, torch.float32).reshape(-1).contiguous()
+        self.u = get(prefix + "u").to(dev, torch.float32).reshape(-1).contiguous()
+        self.norm = get(prefix + "norm").to(dev, torch.float32)
+        self.w_o = get(prefix + "o").to(dev, dt).contiguous()
+
+    def init_random(self, gen, std: float):
+        s, H, N = self.spec, self.hidden, self.spec.size
+        rank = s.decay_rank or max(8, N // 8)
+        t = {n: _rand(gen, N, H, std=std * 4) for n in ("r", "k", "v", "g")}
+        t.update({"mu." + n: torch.rand(H, generator=gen) for n in self.BLENDS})
+        t.update({"w1": _rand(gen, rank, H, std=std * 4), "w2": _rand(gen, N, rank, std=0.5), "w0": _rand(gen, N) - 0.5,
+                  "u": _rand(gen, s.heads, s.dim, std=0.5), "norm": 1.0 + 0.2 * _rand(gen, N), "o": _rand(gen, H, N, std=std)})
+        return t
+
+    def forward(self, x, meta, cache, state):
+        """``x``: the 32-bit rows of the step."""
+        s, ops = self.spec, self.ops
+        T = x.shape[0]
+        mixed = torch.empty(5, T, self.hidden, device=x.device, dtype=self.dtype)
+        ops.token_shift(mixed, x, state[1], self.mu, meta)
+        proj = torch.bmm(mixed[:4], self.w_in_t)                       # [4, T, heads * dim]: r, k, v, gate
+        low = F.linear(mixed[4], self.w1)
+        ops.activation(low, low, "tanh")
+        wl = _linear32(low, self.w2)
+        out = torch.empty(T, s.size, device=x.device, dtype=self.dtype)
+        ops.wkv(out, state[0], proj, wl, self.w0, self.u, self.norm, s, self.eps, meta)
+        return F.linear(out, self.w_o)
 
 
 class GatedDelta:
@@ -481,10 +569,87 @@ class DenseFF:
         return F.linear(up, self.w_down)
 
 
+class RoutedMoE:
+    """``forward`` returns the parts of the mixture's output, (ye, pair_slot, ids, wts, experts, h, shared),
+    which the residual update (``add_normed``) combines: row ``pair_slot[t * top + j]`` of ``ye`` is the
+    output of token t's j-th choice ``ids[t, j]`` (a value >= experts is an identity expert: the token's
+    own input), weighted ``wts[t, j]``; ``shared`` is the shared expert's output or None."""
+
+    def __init__(self, spec: RoutedMoESpec, hidden: int, device, dtype, ops):
+        self.spec, self.hidden, self.device, self.dtype, self.ops = spec, hidden, device, dtype, ops
+        self.w_router = None      # [experts + identity, hidden]
+        self.correction = None    # fp32 [experts + identity]
+        self.w_gu = None          # [E, 2 * ff, hidden]: gate rows, then up rows
+        self.w_down = None        # [E, hidden, ff]
+        self.ws_gu = self.ws_down = None   # the shared expert's [2 * shared_ff, hidden], [hidden, shared_ff]
+
+    def load(self, get, prefix: str):
+        s, dt, dev = self.spec, self.dtype, self.device
+        self.w_router = get(prefix + "router").to(dev, dt).contiguous()
+        self.correction = get(prefix + "correction").to(dev, torch.float32).contiguous()
+        self.w_gu = torch.stack([torch.cat([get(f"{prefix}e{e}.gate"), get(f"{prefix}e{e}.up")], 0)
+                                 for e in range(s.experts)]).to(dev, dt).contiguous()
+        self.w_down = torch.stack([get(f"{prefix}e{e}.down") for e in range(s.experts)]).to(dev, dt).contiguous()
+        if s.shared_ff:
+            self.ws_gu = torch.cat([get(prefix + "shared.gate"), get(prefix + "shared.up")], 0).to(dev, dt).contiguous()
+            self.ws_down = get(prefix + "shared.down").to(dev, dt).contiguous()
+
+    def init_random(self, gen, std: float):
+        s, H = self.spec, self.hidden
+        n = s.experts + s.identity
+        t = {"router": _rand(gen, n, H, std=std * 8), "correction": _rand(gen, n, std=0.1)}
+        for e in range(s.experts):
+            t.update({f"e{e}.gate": _rand(gen, s.ff, H, std=std * 4), f"e{e}.up": _rand(gen, s.ff, H, std=std * 4),
+                      f"e{e}.down": _rand(gen, H, s.ff, std=std * 4)})
+        if s.shared_ff:
+            t.update({"shared.gate": _rand(gen, s.shared_ff, H, std=std * 4), "shared.up": _rand(gen, s.shared_ff, H, std=std * 4),
+                      "shared.down": _rand(gen, H, s.shared_ff, std=std * 4)})
+        return t
+
+    def forward(self, h: torch.Tensor):
+        s, ops = self.spec, self.ops
+        T, dev = h.shape[0], h.device
+        ids = torch.empty(T, s.top, dtype=torch.int32, device=dev)
+        wts = torch.empty(T, s.top, dtype=torch.float32, device=dev)
+        ops.route_topk(ids, wts, _linear32(h, self.w_router), self.correction, s.top, s.scale, s.experts)
+        # the identity experts share one bucket (s.experts) that no GEMM tile serves
+        P, nb = T * s.top, s.experts + (1 if s.identity else 0)
+        tile = MOE_TILE_LARGE if P >= 4 * MOE_TILE_LARGE * nb else MOE_TILE
+        cap = -(-(P + nb * (tile - 1)) // tile) * tile
+        slots = torch.empty(cap, dtype=torch.int32, device=dev)
+        tile_expert = torch.empty(cap // tile, dtype=torch.int32, device=dev)
+        pair_slot = torch.empty(P, dtype=torch.int32, device=dev)
+        ops.moe_align(ids.view(-1), nb, tile, slots, tile_expert, pair_slot)
+        gu = torch.empty(cap, 2 * s.ff, device=dev, dtype=h.dtype)
+        ops.expert_gemm(gu, h, self.w_gu, slots, tile_expert, tile, s.top, False)
+        act = torch.empty(cap, s.ff, device=dev, dtype=h.dtype)
+        ops.activation(act, gu, "silu_mul")
+        ye = torch.empty(cap, self.hidden, device=dev, dtype=h.dtype)
+        ops.expert_gemm(ye, act, self.w_down, slots, tile_expert, tile, 0, False)
+        shared = None
+        if s.shared_ff:
+            g = F.linear(h, self.ws_gu)
+            a = torch.empty(T, s.shared_ff, device=dev, dtype=h.dtype)
+            ops.activation(a, g, "silu_mul")
+            shared = F.linear(a, self.ws_down)
+        return ye, pair_slot, ids, wts, s.experts, h, shared
+
+
+def make_ff(spec, hidden: int, device, dtype, ops):
+    """The weight holder of a feed-forward spec that takes no token ids."""
+    if isinstance(spec, DenseFFSpec):
+        return DenseFF(spec, hidden, device, dtype, ops)
+    if isinstance(spec, RoutedMoESpec):
+        return RoutedMoE(spec, hidden, device, dtype, ops)
+    raise NotImplementedError(type(spec).__name__)
+
+
 def make_mixer(spec, hidden: int, eps: float, device, dtype, ops):
     """The weight holder of a mixer spec (the layer-list designs' common factory)."""
     if isinstance(spec, WindowAttentionSpec):
         return WindowAttention(spec, hidden, eps, device, dtype, ops)
+    if isinstance(spec, WkvSpec):
+        return Wkv(spec, hidden, eps, device, dtype, ops)
     if isinstance(spec, GatedDeltaSpec):
         return GatedDelta(spec, hidden, eps, device, dtype, ops)
     if isinstance(spec, DeltaRuleSpec):

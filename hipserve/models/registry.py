@@ -22,6 +22,7 @@ ARCHITECTURES = {
     "mixtral": ("hipserve.models.llama", "LlamaModel", "hipserve.weights.safetensors_loader:load_hf_weights"),
     "kesirax": ("hipserve.models.kesirax", "KesiraxModel", "hipserve.weights.safetensors_loader:load_named_tensors"),
     "fikizen": ("hipserve.models.fikizen", "FikizenModel", "hipserve.weights.safetensors_loader:load_named_tensors"),
+    "kemavik": ("hipserve.models.kemavik", "KemavikModel", "hipserve.weights.safetensors_loader:load_named_tensors"),
 }
 
 

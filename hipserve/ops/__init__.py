@@ -467,8 +467,21 @@ class ReferenceOps:
     def attn_prepare(self, proj, cache, meta, inv_freq, sp, q_norm, k_norm, eps):
         ref.attn_prepare(proj, cache, meta.positions, meta.slot_mapping, inv_freq, sp, q_norm, k_norm, eps)
 
-    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0):
-        ref.window_attention(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, sp, gate_off, out_scale)
+    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0, lam=0.0, eps=0.0):
+        ref.window_attention(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, sp, gate_off, out_scale, lam, eps)
+
+    def add_normed(self, out, residual, y, w, eps, moe=None):
+        ref.add_normed(out, residual, y, w, eps, moe)
+        return out
+
+    def token_shift(self, out, x, state, mu, meta):
+        ref.token_shift(out, x, state, mu, meta.seq_cu, meta.seq_ctx, meta.seq_state)
+
+    def wkv(self, out, state, proj, wl, w0, u, norm_w, sp, eps, meta):
+        ref.wkv(out, state, proj, wl, w0, u, norm_w, sp, eps, meta.seq_cu, meta.seq_ctx, meta.seq_state)
+
+    def route_topk(self, ids, wts, logits, correction, top, scale, E):
+        ref.route_topk(ids, wts, logits, correction, top, scale, E)
 
     def gated_delta(self, y, state, proj, conv_w, a_log, dt_bias, norm_w, sp, eps, meta):
         ref.gated_delta(y, state[0], state[1], proj, conv_w, a_log, dt_bias, norm_w, sp, eps, meta.seq_cu,

@@ -524,6 +524,8 @@ def expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2):
         if p < 0:
             continue
         e = te[s // tile]
+        if e < 0 or e >= w.shape[0]:   # a tile of the bucket that has no weights (identity experts)
+            continue
         row = p // gather_k if gather_k > 0 else s
         v = w[e].float() @ x[row].float()
         if relu2:
@@ -540,35 +542,49 @@ def _rows_rms(x: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def attn_prepare(proj, cache, positions, slots, inv_freq, sp, q_norm, k_norm, eps):
-    """proj rows = [q | k | v | ...] (after biases). In place on the q columns: the optional
-    whole-projection RMS norm (``sp.qk_norm``) and the rotation; the cache row of slots >= 0
-    gets [rotated keys | values], keys normed alike, values divided by their per-head root
-    mean square when ``sp.v_norm``."""
+    """proj rows = [q | k | v | ...] (after biases), or [q | ...] alone when the layer reads another
+    layer's cache (``sp.kv_from``). In place on the q columns: the optional RMS norm (``sp.qk_norm``:
+    over the whole projection, a weight per element; ``sp.head_norm``: over every head - and map -
+    of ``dim`` elements, one weight of ``dim`` elements for all) and the rotation; the cache row of
+    slots >= 0 gets [keys | values], keys normed and rotated alike, values divided by their per-head
+    root mean square when ``sp.v_norm``."""
     T = proj.shape[0]
     nq, nk, nv = sp.q_size, sp.k_size, sp.v_size
+    own_kv = sp.kv_from is None
     p = proj.float()
-    q, k, v = p[:, :nq], p[:, nq:nq + nk], p[:, nq + nk:nq + nk + nv]
+    q = p[:, :nq]
+    k, v = (p[:, nq:nq + nk], p[:, nq + nk:nq + nk + nv]) if own_kv else (None, None)
     if sp.qk_norm:
         q = _rows_rms(q, eps) * q_norm.float()
+        if own_kv:
+            k = _rows_rms(k, eps) * k_norm.float()
+    q = q.reshape(T, sp.heads * sp.maps, sp.dim)
+    if sp.head_norm:
+        q = _rows_rms(q, eps) * q_norm.float()
+    proj[:, :nq] = partial_rope(q, positions, inv_freq).reshape(T, nq).to(proj.dtype)
+    if not own_kv:
+        return
+    k = k.reshape(T, sp.kv_heads * sp.maps, sp.dim)
+    if sp.head_norm:
         k = _rows_rms(k, eps) * k_norm.float()
-    q = partial_rope(q.reshape(T, sp.heads, sp.dim), positions, inv_freq).reshape(T, nq)
-    k = partial_rope(k.reshape(T, sp.kv_heads, sp.dim), positions, inv_freq).reshape(T, nk)
+    k = partial_rope(k, positions, inv_freq).reshape(T, nk)
     if sp.v_norm:
         v = _rows_rms(v.reshape(T, sp.kv_heads, sp.vdim), eps).reshape(T, nv)
-    proj[:, :nq] = q.to(proj.dtype)
     ok = slots >= 0
     cache.view(-1, cache.shape[-1])[slots[ok]] = torch.cat([k, v], -1).to(cache.dtype)[ok]
 
 
-def window_attention(out, proj, cache, seq_cu, seq_ctx, seq_bt, sp, gate_off, out_scale):
+def window_attention(out, proj, cache, seq_cu, seq_ctx, seq_bt, sp, gate_off, out_scale, lam=0.0, eps=0.0):
     """Per sequence s (rows cu[s]..cu[s+1]-1 at positions ctx[s]-n .. ctx[s]-1): head h scores
     its prepared query against the cached keys of head h // (heads / kv_heads) with
     0 <= pos - j < window; weights exp(s_j) / (sink + sum exp(s_j)); out[t, h * vdim ..] =
-    weighted values * sigmoid(proj[t, gate_off + h]) (gate_off >= 0) * out_scale."""
+    weighted values * sigmoid(proj[t, gate_off + h]) (gate_off >= 0) * out_scale.
+    ``sp.maps`` = 2: query and key heads hold [map 1 | map 2]; the head output is
+    o = a1 - lam * a2 of the two maps' weighted values, o / sqrt(mean(o^2) + eps) * (1 - sp.diff)."""
     bs = cache.shape[1]
     flat = cache.view(-1, cache.shape[-1])
     cu = [int(x) for x in seq_cu]
-    H, G, d, dv, W = sp.heads, sp.kv_heads, sp.dim, sp.vdim, sp.window
+    H, G, M, d, dv, W = sp.heads, sp.kv_heads, sp.maps, sp.dim, sp.vdim, sp.window
     for s in range(len(cu) - 1):
         a, b = cu[s], cu[s + 1]
         if a == b:
@@ -578,9 +594,10 @@ def window_attention(out, proj, cache, seq_cu, seq_ctx, seq_bt, sp, gate_off, ou
         lo = 0 if W <= 0 else max(0, int(pos[0]) - W + 1)
         j = torch.arange(lo, ctx, device=proj.device)
         kv = flat[seq_bt[s].long()[j // bs] * bs + j % bs].float()
-        k = kv[:, :G * d].view(-1, G, d).repeat_interleave(H // G, 1)
-        v = kv[:, G * d:].view(-1, G, dv).repeat_interleave(H // G, 1)
-        q = proj[a:b, :H * d].float().view(b - a, H, d)
+        k = kv[:, :G * M * d].view(-1, G, M * d).repeat_interleave(H // G, 1).reshape(-1, H * M, d)
+        v = kv[:, G * M * d:G * M * d + G * dv].view(-1, G, dv).repeat_interleave(H // G, 1)
+        v = v.repeat_interleave(M, 1)
+        q = proj[a:b, :H * M * d].float().view(b - a, H * M, d)
         sc = torch.einsum("nhd,jhd->hnj", q, k) * sp.scale
         dd = pos[:, None] - j[None]
         ok = (dd >= 0) & ((dd < W) if W > 0 else (dd >= 0))
@@ -591,6 +608,10 @@ def window_attention(out, proj, cache, seq_cu, seq_ctx, seq_bt, sp, gate_off, ou
         e = torch.exp(sc - m)
         den = e.sum(-1, keepdim=True) + (torch.exp(-m) if sp.sink else 0.0)
         o = torch.einsum("hnj,jhv->nhv", e / den, v)
+        if M == 2:
+            o = o.view(b - a, H, 2, dv)
+            o = o[:, :, 0] - lam * o[:, :, 1]
+            o = _rows_rms(o, eps) * (1.0 - sp.diff)
         if gate_off >= 0:
             o = o * torch.sigmoid(proj[a:b, gate_off:gate_off + H].float()).unsqueeze(-1)
         out[a:b] = (o * out_scale).reshape(b - a, H * dv).to(out.dtype)
@@ -677,14 +698,94 @@ def delta_rule(out, S, proj, wl, a_b, w0, norm_w, sp, eps, seq_cu, seq_ctx, seq_
 
 
 def activation(out, x, kind, c0=0.0, c1=0.0):
-    """Elementwise: ``tanh``, or ``xielu`` with c0 = softplus(p), c1 = 1/2 + softplus(q):
-    c0 z^2 + z/2 for z > 0, c1 (exp(z) - 1 - z) + z/2 otherwise."""
+    """Elementwise: ``tanh``; ``relu2`` = max(z, 0)^2; ``xielu`` with c0 = softplus(p),
+    c1 = 1/2 + softplus(q): c0 z^2 + z/2 for z > 0, c1 (exp(z) - 1 - z) + z/2 otherwise;
+    ``silu_mul``: x rows = [gate | up], out = silu(gate) * up (half as wide)."""
     z = x.float()
     if kind == "tanh":
         r = torch.tanh(z)
+    elif kind == "relu2":
+        r = torch.relu(z) ** 2
+    elif kind == "silu_mul":
+        n = z.shape[-1] // 2
+        r = z[..., :n] * torch.sigmoid(z[..., :n]) * z[..., n:]
     elif kind == "xielu":
         zn = z.clamp(max=0.0)
         r = torch.where(z > 0, c0 * z * z + 0.5 * z, c1 * (torch.expm1(zn) - zn) + 0.5 * z)
     else:
         raise ValueError(kind)
     out.copy_(r.to(out.dtype))
+
+
+# ---------------------------------------------------------------------------------
+# residual update with the norm on the sublayer's output, token shift, linear attention
+# with per-channel decays over state slots, softmax router with a selection correction
+
+def add_normed(out, residual, y, w, eps, moe=None):
+    """residual (fp32, in place) += y / sqrt(mean(y^2) + eps) * w; out = residual in out's dtype.
+    With ``moe`` = (ye, pair_slot, ids, wts, E, h, shared) the addend is the mixture's output:
+    y[t] = shared[t] + sum_j wts[t, j] * (ye[pair_slot[t * top + j]] if ids[t, j] < E else h[t])."""
+    if moe is not None:
+        ye, pair_slot, ids, wts, E, h, shared = moe
+        T, top = ids.shape
+        rows = ye.float().index_select(0, pair_slot.long().clamp(min=0)).view(T, top, -1)
+        rows = torch.where((ids < E).unsqueeze(-1), rows, h.float().unsqueeze(1).expand_as(rows))
+        y = (rows * wts.float().unsqueeze(-1)).sum(1)
+        if shared is not None:
+            y = y + shared.float()
+    residual += _rows_rms(y.float(), eps) * w.float()
+    out.copy_(residual.to(out.dtype))
+
+
+def token_shift(out, x, state, mu, seq_cu, seq_ctx, seq_state):
+    """out[s, t] = x[t] + (x[t - 1] - x[t]) * mu[s] for every blend s; the row before a step's first
+    row comes from the sequence's slot (zeros at position 0); the slot gets the step's last row."""
+    cu = [int(v) for v in seq_cu]
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if a == b:
+            continue
+        slot = int(seq_state[s])
+        first = state[slot].clone() if int(seq_ctx[s]) - (b - a) > 0 else torch.zeros_like(state[slot])
+        xs = x[a:b].float()
+        prev = torch.cat([first[None], xs[:-1]], 0)
+        out[:, a:b] = (xs[None] + (prev - xs)[None] * mu.float()[:, None, :]).to(out.dtype)
+        state[slot] = xs[-1]
+
+
+def wkv(out, S, proj, wl, w0, u, norm_w, sp, eps, seq_cu, seq_ctx, seq_state):
+    """proj [4, T, N] = r, k, v and the gate's pre-activation (N = heads * dim), wl the decay
+    bottleneck's output (fp32 [T, N]). Per head: w = exp(-exp(wl + w0)); o = (S + diag(u) k v^T)^T r;
+    S = diag(w) S + k v^T; out = o / rms(o) * norm_w * silu(gate). S [slots, heads, dim(key), dim(value)]."""
+    H, d = sp.heads, sp.dim
+    N = H * d
+    cu = [int(x) for x in seq_cu]
+    for s in range(len(cu) - 1):
+        a0, b0 = cu[s], cu[s + 1]
+        n = b0 - a0
+        if n == 0:
+            continue
+        slot, start = int(seq_state[s]), int(seq_ctx[s]) - n
+        r, k, v = (proj[i, a0:b0].float().view(n, H, d) for i in range(3))
+        g = proj[3, a0:b0].float()
+        w = torch.exp(-torch.exp(wl[a0:b0].float() + w0.float())).view(n, H, d)
+        uu = u.float().view(H, d)
+        st = S[slot].clone() if start > 0 else torch.zeros_like(S[slot])
+        o = torch.empty(n, H, d)
+        for t in range(n):
+            kv = k[t, :, :, None] * v[t, :, None, :]
+            o[t] = torch.einsum("hkv,hk->hv", st + uu[:, :, None] * kv, r[t])
+            st = w[t, :, :, None] * st + kv
+        S[slot] = st
+        out[a0:b0] = (_rows_rms(o, eps).reshape(n, N) * norm_w.float() * (g * torch.sigmoid(g))).to(out.dtype)
+
+
+def route_topk(ids, wts, logits, correction, top, scale, E):
+    """s = softmax(logits) (fp32, over all router outputs); the ``top`` outputs with the largest
+    s + correction are chosen (ties: the lower index); wts = s * scale of the chosen, ids = their
+    index, outputs >= E (experts without weights) all written as E."""
+    s = torch.softmax(logits.float(), -1)
+    c = s + correction.float()
+    order = torch.argsort(-c, dim=-1, stable=True)[:, :top]
+    wts.copy_(s.gather(1, order) * scale)
+    ids.copy_(order.clamp(max=E).to(ids.dtype))
