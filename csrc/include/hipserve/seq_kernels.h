@@ -48,37 +48,58 @@ void launch_mingru_scan(void* y, float* state, const void* proj, const float* b_
                         const int* seq_cu, const int* seq_ctx, const int* seq_state, int nseq, int width, int max_q,
                         bool f32, hipStream_t s);
 
-// out[slot, N] = act(W[e(tile)] [N, K] . x[row(slot)]) over moe_align tiles of `tile` slots.
+// out[slot, N] = act(W[e(tile)] [N, K] . x[row(slot)]) over moe_align tiles of `tile` slots; tiles whose
+// expert is < 0 or >= E (no weights) are skipped.
 void launch_expert_gemm(void* out, const void* x, long x_ld, const void* w, const int* slots, const int* tile_expert,
-                        int ntiles_cap, int tile, int gather_k, int N, int K, bool relu2, bool f32, hipStream_t s);
+                        int ntiles_cap, int tile, int gather_k, int N, int K, bool relu2, int E, bool f32,
+                        hipStream_t s);
+
+// Residual update with the norm on the sublayer's output (group_norm.hip): residual[T, H] (fp32, in place) +=
+// y / sqrt(mean(y^2) + eps) * w; out = residual in the activation type. y null: the addend is a mixture's output,
+// shared (or 0) + sum_j wts[t, j] * (ids[t, j] < E ? ye[pair_slot[t * top + j]] : h[t]).
+void launch_add_normed(void* out, float* residual, const float* w, int T, int H, float eps, const void* y,
+                       const void* ye, const int* pair_slot, const int* ids, const float* wts, int top, int E,
+                       const void* h, const void* shared, bool f32, hipStream_t s);
+
+// Softmax router (router.hip): s = softmax(logits[T, n]); the `top` largest s + correction are chosen (ties: the
+// lower index); ids[T, top] = min(index, E), wts[T, top] = s * scale.
+int route_topk_max_outputs();
+void launch_route_topk(int* ids, float* wts, const float* logits, const float* correction, int T, int n, int top,
+                       float scale, int E, hipStream_t s);
 
 // Window attention on a paged cache [blocks, block_size, kv_heads * dim | kv_heads * vdim] (window_attention.hip).
-// attn_prepare: per row of proj = [q | k | v | ...]: optional whole-projection RMS norm of q and k (q_norm /
-// k_norm null: none), rotate-half rotation of the first 2 * nfreq dims per head, optional per-head unit-rms
-// values; q in place, k / v into cache row slots[t] (>= 0).
+// attn_prepare: per row of proj = [q | k | v | ...]: optional RMS norm of q and k (norm_mode 0: none; 1: over the
+// whole projection, weights per element; 2: per head - and map - of `dim` elements, one weight of `dim` elements),
+// rotate-half rotation of the first 2 * nfreq dims per head, optional per-head unit-rms values; q in place, k / v
+// into cache row slots[t] (>= 0). `maps` query / key maps per head (rows hold heads * maps * dim query and
+// kv_heads * maps * dim key elements). cache null: the rows are [q | ...] and only q is prepared.
 void launch_attn_prepare(void* proj, long ld, void* cache, const long* positions, const long* slots,
-                         const float* inv_freq, int nfreq, int T, int heads, int kv_heads, int dim, int vdim,
-                         const float* q_norm, const float* k_norm, bool v_norm, float eps, bool f32, hipStream_t s);
+                         const float* inv_freq, int nfreq, int T, int heads, int kv_heads, int maps, int dim, int vdim,
+                         const float* q_norm, const float* k_norm, int norm_mode, bool v_norm, float eps, bool f32,
+                         hipStream_t s);
 // Sequences seq0 .. seq1-1 of the step, `tq` tokens per workgroup: keys 0 <= pos - j < window (0: all),
 // weights exp(s_j) / (sink + sum exp), head output times sigmoid(proj[t, gate_off + h]) (gate_off >= 0) and
-// out_scale into out[t * out_ld + h * vdim ..].
+// out_scale into out[t * out_ld + h * vdim ..]. maps = 2 (differential attention): queries and keys hold
+// [map 1 | map 2] per head; the head output is o = a1 - lam a2, o / sqrt(mean(o^2) + eps) * post.
 int window_attention_max_vdim();
 void launch_window_attention(void* out, long out_ld, const void* proj, long proj_ld, const void* cache, int block_size,
                              const int* seq_cu, const int* seq_ctx, const int* seq_bt, int bt_width, int seq0, int seq1,
                              int rows_bound, int tq, int heads, int kv_heads, int dim, int vdim, int gate_off,
-                             float scale, int window, bool sink, float out_scale, bool f32, hipStream_t s);
+                             float scale, int window, bool sink, float out_scale, int maps, float lam, float post,
+                             float eps, bool f32, hipStream_t s);
 
 // bf16 on the matrix cores (window_attention_mfma.hip): 64 (token, head) rows of one key/value head per
 // workgroup, 32-key tiles. nparts > 1 (rows of one token each, rows_bound of them from batch row row_base on):
 // the keys are split into runs of part_keys (a multiple of 32) over ws_acc [nparts, heads, rows_bound, vdim] /
-// ws_ml [.., 2] and merged. out_off: element offset of `out` in its allocation (alignment of the stores).
-bool window_attention_mfma_ok(int dim, int vdim, long out_ld, long out_off);
+// ws_ml [.., 2] and merged (two maps: the workspaces hold 2 * heads "heads"). out_off: element offset of `out`
+// in its allocation (alignment of the stores).
+bool window_attention_mfma_ok(int dim, int vdim, long out_ld, long out_off, int maps);
 void launch_window_attention_mfma(void* out, long out_ld, const void* proj, long proj_ld, const void* cache,
                                   int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt,
                                   int bt_width, int seq0, int seq1, int rows_bound, int heads, int kv_heads, int dim,
                                   int vdim, int gate_off, float scale, int window, bool sink, float out_scale,
-                                  int nparts, int part_keys, float* ws_acc, float* ws_ml, int row_base,
-                                  hipStream_t s);
+                                  int nparts, int part_keys, float* ws_acc, float* ws_ml, int row_base, int maps,
+                                  float lam, float post, float eps, hipStream_t s);
 
 // Delta-rule recurrences over state slots (delta_scan.hip). scratch: fp32, T * (2 * kv_heads * dim +
 // 2 * heads * vdim + 2 * heads) floats for the gated rule, T * 7 * heads * dim for the generalized one.
@@ -92,7 +113,18 @@ void launch_delta_rule(void* out, long out_ld, float* S, const void* proj, long 
                        const float* w0, const float* norm_w, const int* seq_cu, const int* seq_ctx,
                        const int* seq_state, int nseq, int T, float* scratch, int heads, int dim, float eps,
                        float out_scale, bool f32, hipStream_t s);
-// kind 0: tanh; 1: c0 z^2 + z/2 (z > 0), c1 (exp(z) - 1 - z) + z/2 (z <= 0).
+// Token shift: out[nb, T, H] (activation type) = x + (previous row - x) * mu[b] from the 32-bit rows x; a
+// sequence's row before the step comes from state[slot] (zeros at position 0), which then gets the step's last row.
+void launch_token_shift(void* out, const float* x, float* state, const float* mu, const int* seq_cu,
+                        const int* seq_ctx, const int* seq_state, int nseq, int T, int H, int nb, bool f32,
+                        hipStream_t s);
+// Linear attention with per-channel decays: proj [4, T, heads * dim] = r, k, v, gate; wl fp32 [T, heads * dim];
+// scratch: T * (5 * heads * dim + heads) floats.
+void launch_wkv(void* out, float* S, const void* proj, const float* wl, const float* w0, const float* u,
+                const float* norm_w, const int* seq_cu, const int* seq_ctx, const int* seq_state, int nseq, int T,
+                float* scratch, int heads, int dim, float eps, bool f32, hipStream_t s);
+// kind 0: tanh; 1: c0 z^2 + z/2 (z > 0), c1 (exp(z) - 1 - z) + z/2 (z <= 0); 2: max(z, 0)^2;
+// 3: x rows = [gate | up] of `cols` each, out = silu(gate) * up.
 void launch_activation(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, int kind, float c0,
                        float c1, bool f32, hipStream_t s);
 

@@ -5,7 +5,10 @@
 // generalized delta rule (per head, decay w and removal rate a per key channel, unit key u):
 //   S <- diag(w) S - (a * u)(u^T S) + k v^T  (both terms read the old S);  o = S^T r
 //
-// Both scans keep a COLUMN of the state (all key channels of one value channel) in the registers
+// linear attention with a decay per key channel (per head, bonus u for the current token):
+//   o = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T
+//
+// All scans keep a COLUMN of the state (all key channels of one value channel) in the registers
 // of the 16 lanes of a DPP row, dim / 16 key channels each, so a product with the state is a few
 // multiply-adds per lane and a four-step DPP sum; the per-token vectors shared by all columns (k, q / w, a u,
 // u, k, r) are staged through LDS a few tokens at a time. A step that starts at position 0 starts from a zero state.
@@ -349,6 +352,160 @@ __global__ __launch_bounds__(kScanThreads) void delta_rule_scan_kernel(
       if (v0 + cv < dim && k0 + i < dim) Sp[(long)(k0 + i) * dim + v0 + cv] = st[cv][i];
 }
 
+// out[b, t] = x[t] + (x[t - 1] - x[t]) * mu[b] for nb blends of the 32-bit rows x; the row before a sequence's
+// first row of the step comes from its slot of `state` (zeros at position 0).
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_kernel(
+    T* __restrict__ out, const float* __restrict__ x, const float* __restrict__ state, const float* __restrict__ mu,
+    const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx, const int* __restrict__ seq_state, int nseq, int T_,
+    int H, int nb) {
+  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  const int s = find_seq(seq_cu, nseq, t);
+  if (s < 0 || c >= H) return;
+  const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0;
+  const float cur = x[(long)t * H + c];
+  float prev;
+  if (t > r0) prev = x[(long)(t - 1) * H + c];
+  else prev = seq_ctx[s] - n > 0 ? state[(long)seq_state[s] * H + c] : 0.f;
+  const float d = prev - cur;
+  for (int b = 0; b < nb; ++b) stf<T>(out, ((long)b * T_ + t) * H + c, __builtin_fmaf(d, mu[(long)b * H + c], cur));
+}
+
+// The step's last row of every sequence into its slot (after token_shift_kernel has read the old one).
+__global__ __launch_bounds__(256) void shift_state_update_kernel(float* __restrict__ state, const float* __restrict__ x,
+                                                                 const int* __restrict__ seq_cu,
+                                                                 const int* __restrict__ seq_state, int H) {
+  const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  const int r1 = seq_cu[s + 1];
+  if (c >= H || r1 <= seq_cu[s]) return;
+  state[(long)seq_state[s] * H + c] = x[(long)(r1 - 1) * H + c];
+}
+
+// proj [4, T, N] = r, k, v, gate pre-activation (N = heads * dim), wl = decay pre-activation (fp32 [T, N]).
+// pre[t] = [w = exp(-exp(wl + w0)) | k | r | v] as fp32, bonus[t, h] = sum_c r u k over the head's channels.
+template <typename T>
+__global__ __launch_bounds__(256) void wkv_prepare_kernel(
+    float* __restrict__ pre, float* __restrict__ bonus, const T* __restrict__ proj, long T_,
+    const float* __restrict__ wl, const float* __restrict__ w0, const float* __restrict__ u, int heads, int dim) {
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long N = (long)heads * dim;
+  const T* pr = proj + t * N;
+  const T* pk = proj + (T_ + t) * N;
+  const T* pv = proj + (2 * T_ + t) * N;
+  for (int h = wave; h < heads; h += 4) {
+    float b = 0.f;
+    for (int e = lane; e < dim; e += 64) {
+      const int c = h * dim + e;
+      const float r = ldf<T>(pr, c), k = ldf<T>(pk, c);
+      pre[t * 4 * N + c] = expf(-expf(wl[t * N + c] + w0[c]));
+      pre[t * 4 * N + N + c] = k;
+      pre[t * 4 * N + 2 * N + c] = r;
+      pre[t * 4 * N + 3 * N + c] = ldf<T>(pv, c);
+      b = __builtin_fmaf(r * u[c], k, b);
+    }
+    b = wave_sum(b);
+    if (lane == 0) bonus[t * heads + h] = b;
+  }
+}
+
+// Same layout as the delta-rule scans: a state column per 16-lane DPP row, DS key channels per lane. Per token
+// the read-out uses the state BEFORE the update, so the only chain from token to token is one multiply-add per
+// state element; the read-outs' row sums are independent of it.
+template <int DS>
+__global__ __launch_bounds__(kScanThreads) void wkv_scan_kernel(
+    float* __restrict__ o, float* __restrict__ S, const float* __restrict__ pre, const float* __restrict__ bonus,
+    const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx, const int* __restrict__ seq_state, int heads,
+    int dim) {
+  constexpr int DP = kSeg * DS, TB = kTB;
+  __shared__ __attribute__((aligned(16))) float sv[TB][3][DP];  // w, k, r (zero past dim)
+  __shared__ float sb[TB];
+  const int s = blockIdx.z, h = blockIdx.x, zb = blockIdx.y, tid = threadIdx.x;
+  const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0;
+  if (n <= 0) return;
+  const int seg = tid & (kSeg - 1), k0 = seg * DS;
+  const int v0 = zb * kCols + (tid / kSeg) * kCV;   // this lane row's first column
+  const int N = heads * dim;
+  float* Sp = S + (((long)seq_state[s] * heads + h) * dim) * dim;
+  const bool carried = seq_ctx[s] - n > 0;
+  float st[kCV][DS];
+#pragma unroll
+  for (int cv = 0; cv < kCV; ++cv)
+#pragma unroll
+    for (int i = 0; i < DS; ++i)
+      st[cv][i] = (carried && v0 + cv < dim && k0 + i < dim) ? Sp[(long)(k0 + i) * dim + v0 + cv] : 0.f;
+  constexpr int kLd = (TB * DP + kScanThreads - 1) / kScanThreads;
+  float rg[3][kLd], rv[TB][kCV], rb = 0.f;
+  auto fetch = [&](int t0) {
+    const int nt = min(TB, n - t0);
+#pragma unroll
+    for (int it = 0; it < kLd; ++it) {
+      const int i = it * kScanThreads + tid;
+      const int tt = i / DP, k = i % DP;
+      const long row = r0 + t0 + tt;
+      const int c = h * dim + k;
+      const bool in = tt < nt && k < dim;
+#pragma unroll
+      for (int j = 0; j < 3; ++j) rg[j][it] = in ? pre[row * 4 * N + j * N + c] : 0.f;
+    }
+    if (tid < nt) rb = bonus[(long)(r0 + t0 + tid) * heads + h];
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt)
+#pragma unroll
+      for (int cv = 0; cv < kCV; ++cv)
+        rv[tt][cv] = (tt < nt && v0 + cv < dim) ? pre[(long)(r0 + t0 + tt) * 4 * N + 3 * N + h * dim + v0 + cv] : 0.f;
+  };
+  float* po = o + (long)r0 * N + h * dim + v0 + seg;
+  fetch(0);
+  for (int t0 = 0; t0 < n; t0 += TB) {
+    const int nt = min(TB, n - t0);
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kLd; ++it) {
+      const int i = it * kScanThreads + tid;
+      if (i < TB * DP) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) sv[i / DP][j][i % DP] = rg[j][it];
+      }
+    }
+    if (tid < TB) sb[tid] = rb;
+    float val[TB][kCV];
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt)
+#pragma unroll
+      for (int cv = 0; cv < kCV; ++cv) val[tt][cv] = rv[tt][cv];
+    __syncthreads();
+    if (t0 + TB < n) fetch(t0 + TB);
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt) {
+      if (tt < nt) {
+        float w[DS], kk[DS], rr[DS];
+#pragma unroll
+        for (int i = 0; i < DS; ++i) { w[i] = sv[tt][0][k0 + i]; kk[i] = sv[tt][1][k0 + i]; rr[i] = sv[tt][2][k0 + i]; }
+        const float b = sb[tt];
+        float outs[kCV];
+#pragma unroll
+        for (int cv = 0; cv < kCV; ++cv) {
+          float out = 0.f, out2 = 0.f;
+#pragma unroll
+          for (int i = 0; i < DS; ++i) {
+            if (i & 1) out2 = __builtin_fmaf(st[cv][i], rr[i], out2);
+            else out = __builtin_fmaf(st[cv][i], rr[i], out);
+            st[cv][i] = __builtin_fmaf(w[i], st[cv][i], kk[i] * val[tt][cv]);
+          }
+          outs[cv] = __builtin_fmaf(val[tt][cv], b, row_sum(out + out2));
+        }
+        if (seg < kCV && v0 + seg < dim) po[(long)(t0 + tt) * N] = seg == 0 ? outs[0] : outs[kCV - 1];
+      }
+    }
+  }
+#pragma unroll
+  for (int cv = 0; cv < kCV; ++cv)
+#pragma unroll
+    for (int i = 0; i < DS; ++i)
+      if (v0 + cv < dim && k0 + i < dim) Sp[(long)(k0 + i) * dim + v0 + cv] = st[cv][i];
+}
+
 // One wave per (token, head): out = o / rms(o) * w[head * w_stride + e] * act(gate) * scale.
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(
@@ -380,6 +537,8 @@ __global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ out, lo
   const float z = ldf<T>(x, t * x_ld + c);
   float r;
   if (kind == 0) r = tanhf(z);
+  else if (kind == 2) { r = fmaxf(z, 0.f); r *= r; }
+  else if (kind == 3) r = z * sigmoid_f(z) * ldf<T>(x, t * x_ld + cols + c);   // x rows = [gate | up]
   else r = z > 0.f ? c0 * z * z + 0.5f * z : c1 * (expm1f(z) - z) + 0.5f * z;
   stf<T>(out, t * out_ld + c, r);
 }
@@ -392,12 +551,16 @@ __global__ __launch_bounds__(256) void activation_vec_kernel(unsigned short* __r
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= cols8) return;
   const u16x8 z8 = *reinterpret_cast<const u16x8*>(x + t * x_ld + 8 * c);
+  u16x8 u8 = z8;
+  if (kind == 3) u8 = *reinterpret_cast<const u16x8*>(x + t * x_ld + 8 * (cols8 + c));
   u16x8 r8;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const float z = bf16_to_f32(z8[e]);
     float r;
     if (kind == 0) r = tanhf(z);
+    else if (kind == 2) { r = fmaxf(z, 0.f); r *= r; }
+    else if (kind == 3) r = z * sigmoid_f(z) * bf16_to_f32(u8[e]);
     else r = z > 0.f ? c0 * z * z + 0.5f * z : c1 * (expm1f(z) - z) + 0.5f * z;
     r8[e] = f32_to_bf16(r);
   }
@@ -495,6 +658,44 @@ void launch_delta_rule(void* out, long out_ld, float* S, const void* proj, long 
     head_norm_gate<unsigned short>(out, out_ld, o, proj, ld, 4 * N, norm_w, dim, T, heads, dim, eps, false, out_scale,
                                    s);
   }
+}
+
+void launch_token_shift(void* out, const float* x, float* state, const float* mu, const int* seq_cu,
+                        const int* seq_ctx, const int* seq_state, int nseq, int T, int H, int nb, bool f32,
+                        hipStream_t s) {
+  if (nseq <= 0 || T <= 0) return;
+  dim3 grid(T, (H + 255) / 256);
+  if (f32) token_shift_kernel<float><<<grid, 256, 0, s>>>((float*)out, x, state, mu, seq_cu, seq_ctx, seq_state, nseq, T, H, nb);
+  else token_shift_kernel<unsigned short><<<grid, 256, 0, s>>>((unsigned short*)out, x, state, mu, seq_cu, seq_ctx,
+                                                              seq_state, nseq, T, H, nb);
+  shift_state_update_kernel<<<dim3(nseq, (H + 255) / 256), 256, 0, s>>>(state, x, seq_cu, seq_state, H);
+}
+
+void launch_wkv(void* out, float* S, const void* proj, const float* wl, const float* w0, const float* u,
+                const float* norm_w, const int* seq_cu, const int* seq_ctx, const int* seq_state, int nseq, int T,
+                float* scratch, int heads, int dim, float eps, bool f32, hipStream_t s) {
+  if (nseq <= 0 || T <= 0) return;
+  const long N = (long)heads * dim;
+  float* pre = scratch;                   // [T, 4 N]
+  float* bonus = pre + (long)T * 4 * N;   // [T, heads]
+  float* o = bonus + (long)T * heads;     // [T, N]
+  if (f32) wkv_prepare_kernel<float><<<T, 256, 0, s>>>(pre, bonus, (const float*)proj, T, wl, w0, u, heads, dim);
+  else wkv_prepare_kernel<unsigned short><<<T, 256, 0, s>>>(pre, bonus, (const unsigned short*)proj, T, wl, w0, u, heads, dim);
+  dim3 grid(heads, (dim + kCols - 1) / kCols, nseq);
+  switch (ds_of(dim)) {
+#define HS_WK(D)                                                                                                 \
+  case D:                                                                                                        \
+    wkv_scan_kernel<D><<<grid, kScanThreads, 0, s>>>(o, S, pre, bonus, seq_cu, seq_ctx, seq_state, heads, dim);  \
+    break;
+    HS_WK(1) HS_WK(2) HS_WK(4) HS_WK(8) HS_WK(16)
+#undef HS_WK
+  }
+  // the gate's pre-activation is the fourth projection: rows of N from proj + 3 T N
+  if (f32)
+    head_norm_gate<float>(out, N, o, (const float*)proj + 3 * (long)T * N, N, 0, norm_w, dim, T, heads, dim, eps, true, 1.f, s);
+  else
+    head_norm_gate<unsigned short>(out, N, o, (const unsigned short*)proj + 3 * (long)T * N, N, 0, norm_w, dim, T, heads,
+                                   dim, eps, true, 1.f, s);
 }
 
 void launch_activation(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, int kind, float c0,

@@ -1,5 +1,6 @@
-// Expert GEMMs of the table-routed MoE over moe_align tiles: out[slot, :] = act(W[e] . x[row(slot)])
-// where a tile is `tile` consecutive expert-sorted slots of one expert (tile_expert[t], -1 = unused),
+// Expert GEMMs of the mixtures of experts over moe_align tiles: out[slot, :] = act(W[e] . x[row(slot)])
+// where a tile is `tile` consecutive expert-sorted slots of one expert (tile_expert[t]; -1 = unused, and a
+// value >= E, a bucket of pairs whose expert has no weights, is skipped too),
 // row(slot) = slots[slot] / gather_k (the token row of the pair; first GEMM) or the slot itself
 // (second GEMM) and act = squared ReLU or none. Any N and K: edges are bounds-checked. A workgroup
 // computes a [32 slots x 64 columns] block, x and W staged through LDS in K-chunks of 32, fp32
@@ -16,11 +17,11 @@ template <typename T>
 __global__ __launch_bounds__(256) void expert_gemm_kernel(T* __restrict__ out, const T* __restrict__ x, long x_ld,
                                                           const T* __restrict__ w, const int* __restrict__ slots,
                                                           const int* __restrict__ tile_expert, int tile, int gather_k,
-                                                          int N, int K, int relu2) {
+                                                          int N, int K, int relu2, int E) {
   __shared__ float xs[kTM][kTK + 1], ws[kTN][kTK + 1];
   __shared__ long xrow[kTM];
   const int e = tile_expert[(blockIdx.y * kTM) / tile];
-  if (e < 0) return;
+  if (e < 0 || e >= E) return;
   const int tid = threadIdx.x;
   const int slot0 = blockIdx.y * kTM, n0 = blockIdx.x * kTN;
   if (tid < kTM) {
@@ -76,9 +77,9 @@ template <int ST>
 __global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(
     unsigned short* __restrict__ out, const unsigned short* __restrict__ x, long x_ld,
     const unsigned short* __restrict__ w, const int* __restrict__ slots, const int* __restrict__ tile_expert,
-    int gather_k, int N, int K, int relu2) {
+    int gather_k, int N, int K, int relu2, int E) {
   const int e = tile_expert[blockIdx.y];
-  if (e < 0) return;
+  if (e < 0 || e >= E) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int slot0 = blockIdx.y * 16 * ST;
@@ -147,24 +148,24 @@ __global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(
 }  // namespace
 
 void launch_expert_gemm(void* out, const void* x, long x_ld, const void* w, const int* slots, const int* tile_expert,
-                        int ntiles_cap, int tile, int gather_k, int N, int K, bool relu2, bool f32, hipStream_t s) {
+                        int ntiles_cap, int tile, int gather_k, int N, int K, bool relu2, int E, bool f32, hipStream_t s) {
   if (ntiles_cap <= 0) return;
   if (!f32 && K % 8 == 0 && N % 8 == 0 && x_ld % 8 == 0 && (tile == 32 || tile == 64)) {
     dim3 mg((N + 127) / 128, ntiles_cap);
     auto o = (unsigned short*)out;
     auto xi = (const unsigned short*)x, wi = (const unsigned short*)w;
-    if (tile == 32) expert_gemm_mfma_kernel<2><<<mg, 256, 0, s>>>(o, xi, x_ld, wi, slots, tile_expert, gather_k, N, K, relu2);
-    else expert_gemm_mfma_kernel<4><<<mg, 256, 0, s>>>(o, xi, x_ld, wi, slots, tile_expert, gather_k, N, K, relu2);
+    if (tile == 32) expert_gemm_mfma_kernel<2><<<mg, 256, 0, s>>>(o, xi, x_ld, wi, slots, tile_expert, gather_k, N, K, relu2, E);
+    else expert_gemm_mfma_kernel<4><<<mg, 256, 0, s>>>(o, xi, x_ld, wi, slots, tile_expert, gather_k, N, K, relu2, E);
     return;
   }
   dim3 grid((N + kTN - 1) / kTN, (long)ntiles_cap * tile / kTM);
   if (f32)
     expert_gemm_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)x, x_ld, (const float*)w, slots,
-                                                   tile_expert, tile, gather_k, N, K, relu2);
+                                                   tile_expert, tile, gather_k, N, K, relu2, E);
   else
     expert_gemm_kernel<unsigned short><<<grid, 256, 0, s>>>((unsigned short*)out, (const unsigned short*)x, x_ld,
                                                             (const unsigned short*)w, slots, tile_expert, tile,
-                                                            gather_k, N, K, relu2);
+                                                            gather_k, N, K, relu2, E);
 }
 
 }  // namespace hipserve

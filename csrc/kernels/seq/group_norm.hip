@@ -48,7 +48,62 @@ __global__ __launch_bounds__(kNT) void scaled_add_group_rmsnorm_kernel(
   for (int e = tid; e < H; e += kNT) stf<T>(out, t * H + e, r[e] * ginv[e / gs] * w[e]);
 }
 
+// Residual update with the norm on the sublayer's OUTPUT, one workgroup per token row:
+//   y = addend row, or the mixture's output
+//       shared + sum_j wts[t, j] * (ids[t, j] < E ? ye[pair_slot[t * top + j]] : h[t])      (fp32)
+//   residual += y / sqrt(mean(y^2) + eps) * w        (fp32, written back);  out = residual in T
+template <typename T>
+__global__ __launch_bounds__(kNT) void add_normed_kernel(
+    T* __restrict__ out, float* __restrict__ residual, const float* __restrict__ w, int H, float eps,
+    const T* __restrict__ y, const T* __restrict__ ye, const int* __restrict__ pair_slot, const int* __restrict__ ids,
+    const float* __restrict__ wts, int top, int E, const T* __restrict__ h, const T* __restrict__ shared) {
+  extern __shared__ float sm[];  // [H] the addend
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x;
+  float sq = 0.f;
+  float wsum_id = 0.f;  // weight of the token's identity experts
+  if (y == nullptr)
+    for (int j = 0; j < top; ++j)
+      if (ids[t * top + j] >= E) wsum_id += wts[t * top + j];
+  for (int e = tid; e < H; e += kNT) {
+    float v;
+    if (y != nullptr) {
+      v = ldf<T>(y, t * H + e);
+    } else {
+      v = shared != nullptr ? ldf<T>(shared, t * H + e) : 0.f;
+      for (int j = 0; j < top; ++j)
+        if (ids[t * top + j] < E) v = __builtin_fmaf(wts[t * top + j], ldf<T>(ye, (long)pair_slot[t * top + j] * H + e), v);
+      if (wsum_id != 0.f) v = __builtin_fmaf(wsum_id, ldf<T>(h, t * H + e), v);
+    }
+    sm[e] = v;
+    sq += v * v;
+  }
+  sq = block_sum(sq, red);
+  const float inv = 1.f / sqrtf(sq / (float)H + eps);
+  float* r = residual + t * H;
+  for (int e = tid; e < H; e += kNT) {
+    const float v = r[e] + sm[e] * inv * w[e];
+    r[e] = v;
+    stf<T>(out, t * H + e, v);
+  }
+}
+
 }  // namespace
+
+void launch_add_normed(void* out, float* residual, const float* w, int T, int H, float eps, const void* y,
+                       const void* ye, const int* pair_slot, const int* ids, const float* wts, int top, int E,
+                       const void* h, const void* shared, bool f32, hipStream_t s) {
+  if (T <= 0) return;
+  const size_t smem = (size_t)H * sizeof(float);
+  if (f32)
+    add_normed_kernel<float><<<T, kNT, smem, s>>>((float*)out, residual, w, H, eps, (const float*)y, (const float*)ye,
+                                                  pair_slot, ids, wts, top, E, (const float*)h, (const float*)shared);
+  else
+    add_normed_kernel<unsigned short><<<T, kNT, smem, s>>>(
+        (unsigned short*)out, residual, w, H, eps, (const unsigned short*)y, (const unsigned short*)ye, pair_slot, ids,
+        wts, top, E, (const unsigned short*)h, (const unsigned short*)shared);
+}
 
 void launch_scaled_add_group_rmsnorm(void* out, float* residual, const float* w, int T, int H, int groups, float eps,
                                      const void* mix, const float* ls1, const void* y, const int* pair_slot, int top,

@@ -18,6 +18,12 @@
 //      both where P's registers already are and one 16-byte read of the transposed value tile.
 // Rows with few tokens and many keys (decode) split their keys over grid.z; the runs' unnormalised
 // outputs and (max, sum) are merged by window_attention_reduce.
+//
+// DIFF (differential attention): a query / key head holds two maps [map 1 | map 2]. The wave's two
+// 16-row MFMA tiles are then the two MAPS of the same 16 (token, head) rows: each has its own key
+// tile, scores, running (max, sum) and accumulators, and both multiply the one transposed value
+// tile. The epilogue (or the reduce kernel of split rows) forms o = a1 - lam a2 and writes
+// o / sqrt(mean(o^2) + eps) * post.
 #include "seq_common.h"
 #include "hipserve/seq_kernels.h"
 
@@ -47,16 +53,19 @@ HS_DEVICE bool find_tile_rows(const int* __restrict__ seq_cu, int seq0, int seq1
 
 // KS: 32-dim steps of a key head (dim <= 32 KS); NV: 16-dim tiles of a value head (vdim <= 16 NV); MT: 16-row
 // tiles per wave (a workgroup owns 64 MT rows; every key / value operand read from LDS feeds MT MFMAs).
-template <int KS, int NV, int MT>
+template <int KS, int NV, int MT, bool DIFF>
 __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
     unsigned short* __restrict__ out, long out_ld, const unsigned short* __restrict__ proj, long proj_ld,
     const unsigned short* __restrict__ cache, int block_size, const int* __restrict__ seq_cu,
     const int* __restrict__ seq_ctx, const int* __restrict__ seq_bt, int bt_width, int seq0, int seq1, int tq, int hc,
     int hchunks, int heads, int kv_heads, int dim, int vdim, int gate_off, float scale, int window, bool sink,
-    float out_scale, int part_keys, float* __restrict__ ws_acc, float* __restrict__ ws_ml, int row_base, int ws_rows) {
+    float out_scale, int part_keys, float* __restrict__ ws_acc, float* __restrict__ ws_ml, int row_base, int ws_rows,
+    float lam, float post, float eps) {
+  static_assert(!DIFF || MT == 2, "the two row tiles of a wave are the two maps");
   constexpr int kLd = KLd<KS>::v;
-  constexpr int kKF = (KS * 4 + kFT - 1) / kFT, kVF = (NV * 2 + kFT - 1) / kFT;  // 16-byte chunks per thread and tile
-  __shared__ __attribute__((aligned(16))) unsigned short kt[kKeys * kLd];     // [key][dim]
+  constexpr int kMaps = DIFF ? 2 : 1;
+  constexpr int kKF = (kMaps * KS * 4 + kFT - 1) / kFT, kVF = (NV * 2 + kFT - 1) / kFT;  // 16-byte chunks per thread and tile
+  __shared__ __attribute__((aligned(16))) unsigned short kt[kMaps * kKeys * kLd];  // [map][key][dim]
   __shared__ __attribute__((aligned(16))) unsigned short vt[NV * 16 * kVLd];  // [value dim][permuted key]
   int s, tok0;
   if (!find_tile_rows(seq_cu, seq0, seq1, tq, blockIdx.x, s, tok0)) return;
@@ -71,8 +80,8 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
   const int lo_all = window > 0 ? max(0, p_first - window + 1) : 0;
   const int lo = lo_all + blockIdx.z * part_keys;
   const int hi = gridDim.z > 1 ? min(p_last, lo + part_keys - 1) : p_last;
-  const long Dc = (long)kv_heads * (dim + vdim);
-  const long koff = (long)kvh * dim, voff = (long)kv_heads * dim + (long)kvh * vdim;
+  const long Dc = (long)kv_heads * (kMaps * dim + vdim);
+  const long koff = (long)kvh * kMaps * dim, voff = (long)kv_heads * kMaps * dim + (long)kvh * vdim;
   const bool first_part = blockIdx.z == 0;
   const float scale2 = scale * 1.44269504088896341f;
   // this lane's rows: row sr = token sr / hc, head sr % hc of the group
@@ -84,14 +93,14 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
   float m_run[MT], l_run[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int sr = 16 * (wave * MT + mt) + c;
+    const int sr = DIFF ? 16 * wave + c : 16 * (wave * MT + mt) + c;
     const int srt = sr / hc, srh = sr % hc;
     sact[mt] = srt < ntok && srh < nh;
     head[mt] = kvh * group + h0 + (sact[mt] ? srh : 0);
     trow[mt] = r0 + tok0 + (sact[mt] ? srt : 0);
     spos[mt] = p_first + srt;
     s_lo[mt] = window > 0 ? max(0, spos[mt] - window + 1) : 0;
-    const unsigned short* src = proj + trow[mt] * proj_ld + (long)head[mt] * dim;
+    const unsigned short* src = proj + trow[mt] * proj_ld + ((long)head[mt] * kMaps + (DIFF ? mt : 0)) * dim;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       u16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -118,9 +127,10 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
     const long kr = in ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dc : 0;
 #pragma unroll
     for (int i = 0; i < kKF; ++i) {
-      const int ch = fk + kFT * i;
+      const int ch = fk + kFT * i;          // chunk ch % (4 KS) of map ch / (4 KS)
+      const int mp = ch / (KS * 4), cw = ch % (KS * 4);
       kf[i] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (in && ch < kchunks) kf[i] = *reinterpret_cast<const u16x8*>(cache + kr + koff + 8 * ch);
+      if (in && mp < kMaps && cw < kchunks) kf[i] = *reinterpret_cast<const u16x8*>(cache + kr + koff + mp * dim + 8 * cw);
     }
 #pragma unroll
     for (int i = 0; i < kVF; ++i) {
@@ -135,7 +145,8 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < kKF; ++i) {
       const int ch = fk + kFT * i;
-      if (ch < KS * 4) *reinterpret_cast<u16x8*>(kt + fkey * kLd + 8 * ch) = kf[i];
+      if (ch < kMaps * KS * 4)
+        *reinterpret_cast<u16x8*>(kt + (ch / (KS * 4)) * kKeys * kLd + fkey * kLd + 8 * (ch % (KS * 4))) = kf[i];
     }
 #pragma unroll
     for (int i = 0; i < kVF; ++i) {
@@ -155,10 +166,19 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
     for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
-        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8*>(kt + (16 * nt + c) * kLd + 32 * ks + 8 * g));
+        if constexpr (DIFF) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          sc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[mt][ks], sc[mt][nt], 0, 0, 0);
+          for (int mt = 0; mt < MT; ++mt) {  // map mt: its own key tile
+            const bf16x8 a = __builtin_bit_cast(
+                bf16x8, *reinterpret_cast<const u16x8*>(kt + mt * kKeys * kLd + (16 * nt + c) * kLd + 32 * ks + 8 * g));
+            sc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[mt][ks], sc[mt][nt], 0, 0, 0);
+          }
+        } else {
+          const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8*>(kt + (16 * nt + c) * kLd + 32 * ks + 8 * g));
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            sc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[mt][ks], sc[mt][nt], 0, 0, 0);
+        }
       }
     }
     bf16x8 pb8[MT];
@@ -216,6 +236,47 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
     }
   }
   // lane (c, g) holds value dims 16 j + 4 g .. + 3 of its rows
+  if constexpr (DIFF) {
+    if (!sact[0]) return;
+    if (gridDim.z > 1) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {  // the runs of map mt live under "head" 2 head + mt
+        const long wrow = ((long)blockIdx.z * heads * 2 + head[0] * 2 + mt) * ws_rows + (trow[0] - row_base);
+        if (g == 0) { ws_ml[2 * wrow] = m_run[mt]; ws_ml[2 * wrow + 1] = l_run[mt]; }
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+          const int d = 16 * j + 4 * g;
+          if (d < vdim) *reinterpret_cast<f32x4*>(ws_acc + wrow * vdim + d) = acc[mt][j];
+        }
+      }
+      return;
+    }
+    const float i0 = l_run[0] > 0.f ? 1.f / l_run[0] : 0.f, i1 = l_run[1] > 0.f ? lam / l_run[1] : 0.f;
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float o = acc[0][j][e] * i0 - acc[1][j][e] * i1;  // dims past vdim are zero (zero value rows)
+        acc[0][j][e] = o;
+        ss += o * o;
+      }
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    float f = out_scale * post / sqrtf(ss / (float)vdim + eps);
+    if (gate_off >= 0) f *= sigmoid_f(bf16_to_f32(proj[trow[0] * proj_ld + gate_off + head[0]]));
+    unsigned short* dst = out + trow[0] * out_ld + (long)head[0] * vdim;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int d = 16 * j + 4 * g;
+      if (d >= vdim) continue;
+      u16x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16(acc[0][j][e] * f);
+      *reinterpret_cast<u16x4*>(dst + d) = o;
+    }
+    return;
+  }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     if (!sact[mt]) continue;
@@ -273,24 +334,71 @@ __global__ __launch_bounds__(128) void window_attention_reduce_kernel(
   }
 }
 
-template <int KS, int NV, int MT>
+// Two maps per head: the runs of map m of head h sit under workspace head 2 h + m (of 2 heads). Each map's runs
+// are merged as above, then o = a1 - lam a2 and out = o / sqrt(mean(o^2) + eps) * post * gate * out_scale.
+__global__ __launch_bounds__(128) void window_attention_diff_reduce_kernel(
+    unsigned short* __restrict__ out, long out_ld, const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
+    const unsigned short* __restrict__ proj, long proj_ld, int gate_off, int nparts, int heads, int ws_rows,
+    int row_base, int vdim, float out_scale, float lam, float post, float eps) {
+  __shared__ float sc[2][kMaxRuns];
+  __shared__ float red[16];
+  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  {  // wave m: map m, run p on lane p
+    const long w = ((long)min(lane, nparts - 1) * heads * 2 + 2 * h + wave) * ws_rows + r;
+    const float m = lane < nparts ? ws_ml[2 * w] : -INFINITY;
+    const float l = lane < nparts ? ws_ml[2 * w + 1] : 0.f;
+    const float M = wave_max(m);
+    const float e = m > -INFINITY ? __builtin_amdgcn_exp2f(m - M) : 0.f;
+    const float L = wave_sum(l * e);
+    sc[wave][lane] = L > 0.f ? e * (wave == 1 ? lam : 1.f) / L : 0.f;
+  }
+  __syncthreads();
+  float o[2] = {0.f, 0.f};  // vdim <= 256: dims tid, tid + 128
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int d = tid + 128 * i;
+    if (d < vdim) {
+      for (int p = 0; p < nparts; ++p) {
+        const long w0 = ((long)p * heads * 2 + 2 * h) * ws_rows + r;
+        o[i] += ws_acc[w0 * vdim + d] * sc[0][p] - ws_acc[(w0 + ws_rows) * vdim + d] * sc[1][p];
+      }
+      ss += o[i] * o[i];
+    }
+  }
+  ss = block_sum(ss, red);
+  float f = out_scale * post / sqrtf(ss / (float)vdim + eps);
+  const long trow = row_base + r;
+  if (gate_off >= 0) f *= sigmoid_f(bf16_to_f32(proj[trow * proj_ld + gate_off + h]));
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int d = tid + 128 * i;
+    if (d < vdim) out[trow * out_ld + (long)h * vdim + d] = f32_to_bf16(o[i] * f);
+  }
+}
+
+template <int KS, int NV, int MT, bool DIFF>
 void launch_mfma(unsigned short* out, long out_ld, const unsigned short* proj, long proj_ld, const unsigned short* cache,
                  int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt, int bt_width, int seq0,
                  int seq1, int rows_bound, int heads, int kv_heads, int dim, int vdim, int gate_off, float scale,
                  int window, bool sink, float out_scale, int nparts, int part_keys, float* ws_acc, float* ws_ml,
-                 int row_base, hipStream_t s) {
+                 int row_base, float lam, float post, float eps, hipStream_t s) {
   const int group = heads / kv_heads;
-  const int rows = kRows * MT;
+  const int rows = DIFF ? kRows : kRows * MT;
   const int hc = min(group, rows);
   const int hchunks = (group + hc - 1) / hc;
   // split rows (decode): one token per workgroup; else as many consecutive tokens as fit the rows
   const int tq = nparts > 1 ? 1 : rows / hc;
   dim3 grid(rows_bound / tq + (seq1 - seq0), kv_heads * hchunks, nparts);
-  window_attention_mfma_kernel<KS, NV, MT><<<grid, kThreads, 0, s>>>(
+  window_attention_mfma_kernel<KS, NV, MT, DIFF><<<grid, kThreads, 0, s>>>(
       out, out_ld, proj, proj_ld, cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1, tq, hc, hchunks,
       heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale, part_keys, ws_acc, ws_ml, row_base,
-      rows_bound);
-  if (nparts > 1)
+      rows_bound, lam, post, eps);
+  if (nparts > 1 && DIFF)
+    window_attention_diff_reduce_kernel<<<dim3(rows_bound, heads), 128, 0, s>>>(
+        out, out_ld, ws_acc, ws_ml, proj, proj_ld, gate_off, nparts, heads, rows_bound, row_base, vdim, out_scale, lam,
+        post, eps);
+  else if (nparts > 1)
     window_attention_reduce_kernel<<<dim3(rows_bound, heads), 128, 0, s>>>(out, out_ld, ws_acc, ws_ml, proj, proj_ld,
                                                                          gate_off, nparts, heads, rows_bound, row_base,
                                                                          vdim, out_scale);
@@ -298,28 +406,35 @@ void launch_mfma(unsigned short* out, long out_ld, const unsigned short* proj, l
 
 }  // namespace
 
-bool window_attention_mfma_ok(int dim, int vdim, long out_ld, long out_off) {
-  return dim % 8 == 0 && vdim % 8 == 0 && dim <= 256 && vdim <= 256 && out_ld % 4 == 0 && out_off % 4 == 0;
+bool window_attention_mfma_ok(int dim, int vdim, long out_ld, long out_off, int maps) {
+  const int cap = maps == 2 ? 128 : 256;  // two maps: the kernel variants with two row tiles per wave
+  return dim % 8 == 0 && vdim % 8 == 0 && dim <= cap && vdim <= cap && out_ld % 4 == 0 && out_off % 4 == 0 &&
+         (maps == 1 || maps == 2);
 }
 
 void launch_window_attention_mfma(void* out, long out_ld, const void* proj, long proj_ld, const void* cache,
                                   int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt,
                                   int bt_width, int seq0, int seq1, int rows_bound, int heads, int kv_heads, int dim,
                                   int vdim, int gate_off, float scale, int window, bool sink, float out_scale,
-                                  int nparts, int part_keys, float* ws_acc, float* ws_ml, int row_base,
-                                  hipStream_t s) {
+                                  int nparts, int part_keys, float* ws_acc, float* ws_ml, int row_base, int maps,
+                                  float lam, float post, float eps, hipStream_t s) {
   if (seq1 <= seq0 || rows_bound <= 0) return;
-#define HS_WA(KS, NV, MT)                                                                                           \
-  launch_mfma<KS, NV, MT>((unsigned short*)out, out_ld, (const unsigned short*)proj, proj_ld,                        \
-                          (const unsigned short*)cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1,    \
-                          rows_bound, heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale, nparts,   \
-                          part_keys, ws_acc, ws_ml, row_base, s)
+#define HS_WA(KS, NV, MT, DIFF)                                                                                     \
+  launch_mfma<KS, NV, MT, DIFF>((unsigned short*)out, out_ld, (const unsigned short*)proj, proj_ld,                  \
+                                (const unsigned short*)cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0,    \
+                                seq1, rows_bound, heads, kv_heads, dim, vdim, gate_off, scale, window, sink,          \
+                                out_scale, nparts, part_keys, ws_acc, ws_ml, row_base, lam, post, eps, s)
   // two row tiles per wave where a prompt portion brings enough rows and the accumulators fit the registers
   const int ks = (dim + 31) / 32, nv = (vdim + 15) / 16;
+  if (maps == 2) {
+    if (ks <= 2 && nv <= 4) HS_WA(2, 4, 2, true);
+    else HS_WA(4, 8, 2, true);
+    return;
+  }
   const bool wide = nparts == 1 && (long)rows_bound * (heads / kv_heads) >= 128 * (long)(seq1 - seq0);
-  if (ks <= 2 && nv <= 4) { if (wide) HS_WA(2, 4, 2); else HS_WA(2, 4, 1); }
-  else if (ks <= 4 && nv <= 8) { if (wide) HS_WA(4, 8, 2); else HS_WA(4, 8, 1); }
-  else HS_WA(8, 16, 1);
+  if (ks <= 2 && nv <= 4) { if (wide) HS_WA(2, 4, 2, false); else HS_WA(2, 4, 1, false); }
+  else if (ks <= 4 && nv <= 8) { if (wide) HS_WA(4, 8, 2, false); else HS_WA(4, 8, 1, false); }
+  else HS_WA(8, 16, 1, false);
 #undef HS_WA
 }
 

@@ -8,6 +8,7 @@
 
 #include "hipserve/kernels.h"
 #include "hipserve/seq_kernels.h"
+#include "hipserve/seq_shared_bindings.h"
 
 namespace {
 
@@ -171,38 +172,8 @@ void mingru_scan(at::Tensor& y, at::Tensor& state, const at::Tensor& proj, const
                                seq_state.data_ptr<int>(), nseq, width, max_q, f32, cur_stream());
 }
 
-void moe_align(const at::Tensor& ids, int64_t E, int64_t tile, at::Tensor& slots, at::Tensor& tile_expert,
-               at::Tensor& pair_slot) {
-  CHECK_DEV(ids); CHECK_I32(ids); CHECK_I32(slots); CHECK_I32(tile_expert); CHECK_I32(pair_slot);
-  TORCH_CHECK(E >= 1 && E <= 128, "moe_align: at most 128 experts");
-  TORCH_CHECK(tile == 16 || tile == 32 || tile == 64 || tile == 128 || tile == 256);
-  const int npairs = ids.numel();
-  TORCH_CHECK(slots.numel() >= npairs + E * (tile - 1) && slots.numel() % tile == 0,
-              "slots capacity must cover padding and be a multiple of the tile");
-  TORCH_CHECK(tile_expert.numel() * tile >= slots.numel() && pair_slot.numel() >= npairs);
-  c10::hip::HIPGuardMasqueradingAsCUDA g(ids.device());
-  const int nb = hipserve::moe_align_blocks(npairs);
-  at::Tensor scratch = at::empty({(long)(nb > 1 ? nb : 0) * 128 + 1}, ids.options());  // [hist | tile count]
-  hipserve::launch_moe_align(ids.data_ptr<int>(), npairs, E, tile, slots.data_ptr<int>(), slots.numel(),
-                             tile_expert.data_ptr<int>(), tile_expert.numel(),
-                             scratch.data_ptr<int>() + (scratch.numel() - 1), pair_slot.data_ptr<int>(), nullptr,
-                             cur_stream(), nb > 1 ? scratch.data_ptr<int>() : nullptr);
-}
-
-void expert_gemm(at::Tensor& out, const at::Tensor& x, const at::Tensor& w, const at::Tensor& slots,
-                 const at::Tensor& tile_expert, int64_t tile, int64_t gather_k, bool relu2) {
-  CHECK_DEV(x); CHECK_CONTIG(out); CHECK_CONTIG(w); CHECK_I32(slots); CHECK_I32(tile_expert);
-  const bool f32 = is_f32(x, "expert_gemm");
-  TORCH_CHECK(out.scalar_type() == x.scalar_type() && w.scalar_type() == x.scalar_type());
-  TORCH_CHECK(w.dim() == 3 && x.dim() == 2 && x.stride(1) == 1 && out.dim() == 2);
-  const long N = w.size(1), K = w.size(2), cap = slots.numel();
-  TORCH_CHECK(x.size(1) == K && out.size(1) == N && out.size(0) >= cap);
-  TORCH_CHECK(tile % 32 == 0 && cap % tile == 0 && tile_expert.numel() * tile >= cap, "tiles of a multiple of 32 slots");
-  TORCH_CHECK(gather_k > 0 || x.size(0) >= cap, "ungathered x needs one row per slot");
-  c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
-  hipserve::launch_expert_gemm(out.data_ptr(), x.data_ptr(), x.stride(0), w.data_ptr(), slots.data_ptr<int>(),
-                               tile_expert.data_ptr<int>(), cap / tile, tile, gather_k, N, K, relu2, f32, cur_stream());
-}
+using hipserve_shared::expert_gemm;
+using hipserve_shared::moe_align;
 
 }  // namespace
 

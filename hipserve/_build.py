@@ -39,15 +39,17 @@ HIP_FLAGS = [
 
 # kernel libraries: name -> (shared object, kernel sources, host bindings). "core" is every
 # dense-transformer / sampling / quantisation kernel; "seq" the latent-attention / minGRU / table-MoE
-# kernels of the layer-list decoders (plus the expert alignment of moe.hip); "delta" their window
-# attention, delta-rule recurrences and activations. The residual + norm kernel is linked into both
-# of the latter, so a model of those designs builds only what it runs.
+# kernels of the layer-list decoders (plus the expert alignment of moe.hip); "delta" their window and
+# differential attention, delta-rule and decayed linear-attention recurrences, softmax router and
+# activations. The residual + norm kernels, the expert alignment and the expert GEMMs are linked into
+# both of the latter, so a model of those designs builds only what it runs.
 LIBS = {
     "core": ("_C.so", ["kernels/*.hip"], "torch_bindings.cpp"),
     "seq": ("_C_seq.so", ["kernels/seq/group_norm.hip", "kernels/seq/latent_attention*.hip", "kernels/seq/mingru.hip",
                           "kernels/seq/expert_ffn.hip", "kernels/moe.hip"], "seq_bindings.cpp"),
     "delta": ("_C_delta.so", ["kernels/seq/group_norm.hip", "kernels/seq/window_attention*.hip",
-                              "kernels/seq/delta_scan.hip"], "seq_delta_bindings.cpp"),
+                              "kernels/seq/delta_scan.hip", "kernels/seq/router.hip", "kernels/seq/expert_ffn.hip",
+                              "kernels/moe.hip"], "seq_delta_bindings.cpp"),
 }
 
 

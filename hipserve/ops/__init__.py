@@ -271,28 +271,32 @@ class KernelOps:
         self._seq.mingru_scan(y, state, proj, b_z, b_x, meta.seq_cu, meta.seq_ctx, meta.seq_state, meta.max_q)
 
     def attn_prepare(self, proj, cache, meta, inv_freq, sp, q_norm, k_norm, eps):
-        self._delta.attn_prepare(proj, cache, meta.positions, meta.slot_mapping, inv_freq, sp.heads, sp.kv_heads,
-                               sp.dim, sp.vdim, q_norm if sp.qk_norm else None, k_norm if sp.qk_norm else None,
-                               sp.v_norm, eps)
+        mode = 1 if sp.qk_norm else 2 if sp.head_norm else 0
+        own_kv = sp.kv_from is None   # else the layer reads another layer's cache: only q is prepared
+        self._delta.attn_prepare(proj, cache if own_kv else None, meta.positions, meta.slot_mapping, inv_freq, sp.heads,
+                                 sp.kv_heads, sp.maps, sp.dim, sp.vdim, q_norm if mode else None,
+                                 k_norm if mode and own_kv else None, mode, sp.v_norm, eps)
 
     WINDOW_PREFILL_TQ = 4  # tokens per workgroup of a prompt portion (x the query heads of one key/value head)
     # bf16 runs the MFMA kernel (HIPSERVE_WINDOW_MFMA=0: the generic kernel, as fp32 does)
     WINDOW_MFMA = os.environ.get("HIPSERVE_WINDOW_MFMA", "1") != "0"
     WINDOW_DECODE_RUN = 128  # keys per run of a decode row (a multiple of 32)
 
-    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0):
+    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0, lam=0.0, eps=0.0):
         """Prompt portions (the step's first sequences) run several tokens per workgroup, decode
-        rows one token per workgroup."""
+        rows one token per workgroup. Two maps per head (``sp.maps`` = 2): ``lam`` weighs the second
+        map, the head output is divided by its root mean square (``eps``) and scaled by 1 - ``sp.diff``."""
         nseq = meta.seq_ctx.shape[0]
         nd = meta.num_decode
         npf, Tp = nseq - nd, meta.num_prefill_tokens
+        diff = (sp.maps, lam, 1.0 - sp.diff, eps)
         if (proj.dtype == torch.bfloat16 and self.WINDOW_MFMA
-                and self._delta.window_attention_mfma_ok(sp.dim, sp.vdim, out.stride(0), out.storage_offset())):
+                and self._delta.window_attention_mfma_ok(sp.dim, sp.vdim, out.stride(0), out.storage_offset(), sp.maps)):
             # bf16: the matrix-core kernel; decode rows split their keys into runs merged by a reduce kernel
             args = (sp.heads, sp.kv_heads, sp.dim, sp.vdim, gate_off, sp.scale, sp.window, sp.sink, out_scale)
             if npf:
                 self._delta.window_attention_mfma(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, 0, npf, Tp,
-                                                *args, 1, 0, None, None, 0)
+                                                *args, 1, 0, None, None, 0, *diff)
             if nd:
                 span = min(sp.window, meta.max_ctx or sp.window) if sp.window > 0 else meta.max_ctx
                 part = self.WINDOW_DECODE_RUN
@@ -301,16 +305,16 @@ class KernelOps:
                 nparts = max(1, -(-span // part))
                 ws_acc = ws_ml = None
                 if nparts > 1:
-                    ws_acc = torch.empty(nparts, sp.heads, nd, sp.vdim, device=proj.device, dtype=torch.float32)
-                    ws_ml = torch.empty(nparts, sp.heads, nd, 2, device=proj.device, dtype=torch.float32)
+                    ws_acc = torch.empty(nparts, sp.heads * sp.maps, nd, sp.vdim, device=proj.device, dtype=torch.float32)
+                    ws_ml = torch.empty(nparts, sp.heads * sp.maps, nd, 2, device=proj.device, dtype=torch.float32)
                 self._delta.window_attention_mfma(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, npf, nseq, nd,
-                                                *args, nparts, part, ws_acc, ws_ml, Tp)
+                                                *args, nparts, part, ws_acc, ws_ml, Tp, *diff)
             return
         for s0, s1, rows, tq in ((0, npf, Tp, self.WINDOW_PREFILL_TQ), (npf, nseq, nd, 1)):
             if s1 > s0:
                 self._delta.window_attention(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, s0, s1, rows, tq,
                                            sp.heads, sp.kv_heads, sp.dim, sp.vdim, gate_off, sp.scale, sp.window,
-                                           sp.sink, out_scale)
+                                           sp.sink, out_scale, *diff)
 
     def gated_delta(self, y, state, proj, conv_w, a_log, dt_bias, norm_w, sp, eps, meta):
         T = proj.shape[0]
@@ -324,15 +328,44 @@ class KernelOps:
         self._delta.delta_rule(out, state[0], proj, wl, a_b, w0, norm_w, meta.seq_cu, meta.seq_ctx, meta.seq_state,
                              scratch, sp.heads, sp.dim, eps, out_scale)
 
-    ACTIVATIONS = {"tanh": 0, "xielu": 1}
+    ACTIVATIONS = {"tanh": 0, "xielu": 1, "relu2": 2, "silu_mul": 3}
 
     def activation(self, out, x, kind, c0=0.0, c1=0.0):
         self._delta.activation(out, x, self.ACTIVATIONS[kind], c0, c1)
         return out
 
+    def add_normed(self, out, residual, y, w, eps, moe=None):
+        if moe is None:
+            self._delta.add_normed(out, residual, w, eps, y, None, None, None, None, 0, None, None)
+        else:
+            ye, pair_slot, ids, wts, E, h, shared = moe
+            self._delta.add_normed(out, residual, w, eps, None, ye, pair_slot, ids, wts, E, h, shared)
+        return out
+
+    def token_shift(self, out, x, state, mu, meta):
+        self._delta.token_shift(out, x, state, mu, meta.seq_cu, meta.seq_ctx, meta.seq_state)
+
+    def wkv(self, out, state, proj, wl, w0, u, norm_w, sp, eps, meta):
+        scratch = torch.empty(proj.shape[1] * (5 * sp.size + sp.heads), device=proj.device, dtype=torch.float32)
+        self._delta.wkv(out, state, proj, wl, w0, u, norm_w, meta.seq_cu, meta.seq_ctx, meta.seq_state, scratch,
+                        sp.heads, sp.dim, eps)
+
+    ROUTER_MAX_OUTPUTS = 256
+
+    def route_topk(self, ids, wts, logits, correction, top, scale, E):
+        if logits.shape[1] > self.ROUTER_MAX_OUTPUTS:   # more router outputs than a wave holds: device-side torch ops
+            ref.route_topk(ids, wts, logits, correction, top, scale, E)
+            return
+        self._delta.route_topk(ids, wts, logits.contiguous(), correction, top, scale, E)
+
+    @property
+    def _moe_lib(self):
+        """The library whose copy of the expert alignment and expert GEMMs runs (the one the model loads anyway)."""
+        return self._delta if self.norm_library == "delta" else self._seq
+
     def moe_align(self, experts, E, tile, slots, tile_expert, pair_slot):
         if E <= 128:
-            self._seq.moe_align(experts, E, tile, slots, tile_expert, pair_slot)
+            self._moe_lib.moe_align(experts, E, tile, slots, tile_expert, pair_slot)
             return
         # more experts than the alignment kernel's LDS tables hold: the same layout from device-side
         # sort / scan ops (no host round trip)
@@ -353,7 +386,7 @@ class KernelOps:
         tile_expert.copy_(torch.where(te < E, te, torch.full_like(te, -1)).to(torch.int32))
 
     def expert_gemm(self, out, x, w, slots, tile_expert, tile, gather_k, relu2):
-        self._seq.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2)
+        self._moe_lib.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2)
 
 
 class ReferenceOps:
