@@ -49,9 +49,10 @@ void launch_mingru_scan(void* y, float* state, const void* proj, const float* b_
                         bool f32, hipStream_t s);
 
 // out[slot, N] = act(W[e(tile)] [N, K] . x[row(slot)]) over moe_align tiles of `tile` slots; tiles whose
-// expert is < 0 or >= E (no weights) are skipped.
+// expert is < 0 or >= E (no weights) are skipped. act 0: none, 1: squared ReLU, 2: W[e] = [gate rows; up rows]
+// and out[slot, N / 2] = silu(gate) * up.
 void launch_expert_gemm(void* out, const void* x, long x_ld, const void* w, const int* slots, const int* tile_expert,
-                        int ntiles_cap, int tile, int gather_k, int N, int K, bool relu2, int E, bool f32,
+                        int ntiles_cap, int tile, int gather_k, int N, int K, int act, int E, bool f32,
                         hipStream_t s);
 
 // Residual update with the norm on the sublayer's output (group_norm.hip): residual[T, H] (fp32, in place) +=

@@ -32,7 +32,7 @@ inline void moe_align(const at::Tensor& ids, int64_t E, int64_t tile, at::Tensor
 }
 
 inline void expert_gemm(at::Tensor& out, const at::Tensor& x, const at::Tensor& w, const at::Tensor& slots,
-                        const at::Tensor& tile_expert, int64_t tile, int64_t gather_k, bool relu2) {
+                        const at::Tensor& tile_expert, int64_t tile, int64_t gather_k, int64_t act) {
   auto i32 = [](const at::Tensor& t) { return t.scalar_type() == at::kInt && t.is_contiguous(); };
   TORCH_CHECK(x.is_cuda() && out.is_contiguous() && w.is_contiguous() && i32(slots) && i32(tile_expert));
   TORCH_CHECK(x.scalar_type() == at::kFloat || x.scalar_type() == at::kBFloat16, "expert_gemm: bf16 or fp32 activations");
@@ -40,12 +40,13 @@ inline void expert_gemm(at::Tensor& out, const at::Tensor& x, const at::Tensor& 
   TORCH_CHECK(out.scalar_type() == x.scalar_type() && w.scalar_type() == x.scalar_type());
   TORCH_CHECK(w.dim() == 3 && x.dim() == 2 && x.stride(1) == 1 && out.dim() == 2);
   const long N = w.size(1), K = w.size(2), cap = slots.numel();
-  TORCH_CHECK(x.size(1) == K && out.size(1) == N && out.size(0) >= cap);
+  TORCH_CHECK(act >= 0 && act <= 2 && (act != 2 || N % 2 == 0), "expert_gemm: act 0 (none), 1 (relu^2), 2 (silu gate)");
+  TORCH_CHECK(x.size(1) == K && out.size(1) == (act == 2 ? N / 2 : N) && out.size(0) >= cap);
   TORCH_CHECK(tile % 32 == 0 && cap % tile == 0 && tile_expert.numel() * tile >= cap, "tiles of a multiple of 32 slots");
   TORCH_CHECK(gather_k > 0 || x.size(0) >= cap, "ungathered x needs one row per slot");
   c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
   hipserve::launch_expert_gemm(out.data_ptr(), x.data_ptr(), x.stride(0), w.data_ptr(), slots.data_ptr<int>(),
-                               tile_expert.data_ptr<int>(), cap / tile, tile, gather_k, N, K, relu2, w.size(0), f32,
+                               tile_expert.data_ptr<int>(), cap / tile, tile, gather_k, N, K, act, w.size(0), f32,
                                c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
 }
 

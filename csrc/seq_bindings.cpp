@@ -194,7 +194,7 @@ TORCH_LIBRARY(hipserve_seq, m) {
         "Tensor seq_ctx, Tensor seq_state, int max_q) -> ()");
   m.def("moe_align(Tensor ids, int E, int tile, Tensor(a!) slots, Tensor(b!) tile_expert, Tensor(c!) pair_slot) -> ()");
   m.def("expert_gemm(Tensor(a!) out, Tensor x, Tensor w, Tensor slots, Tensor tile_expert, int tile, int gather_k, "
-        "bool relu2) -> ()");
+        "int act) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(hipserve_seq, CUDA, m) {

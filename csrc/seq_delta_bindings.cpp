@@ -342,7 +342,7 @@ TORCH_LIBRARY(hipserve_delta, m) {
   m.def("route_topk(Tensor(a!) ids, Tensor(b!) wts, Tensor logits, Tensor correction, int top, float scale, int E) -> ()");
   m.def("moe_align(Tensor ids, int E, int tile, Tensor(a!) slots, Tensor(b!) tile_expert, Tensor(c!) pair_slot) -> ()");
   m.def("expert_gemm(Tensor(a!) out, Tensor x, Tensor w, Tensor slots, Tensor tile_expert, int tile, int gather_k, "
-        "bool relu2) -> ()");
+        "int act) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(hipserve_delta, CUDA, m) {

@@ -2,7 +2,8 @@
 sizes that resemble a real model's layers, each beside the closest existing family at equal
 size: Kesirax beside a Mixtral-style model (sliding-window attention + MoE feed-forward),
 Fikizen beside a dense sliding-window model (grouped-query attention + gated dense
-feed-forward). Random-init weights, synthetic prompts, a few layers of each (the per-layer
+feed-forward), Kemavik beside Fikizen (the other design that mixes attention layers with
+linear recurrences; its attention has no window). Random-init weights, synthetic prompts, a few layers of each (the per-layer
 cost is what is compared). ``--layer-models`` picks the models; the ratios are given per pair.
 
 Per size and model, through the engine's own scheduler and step function:
@@ -75,8 +76,27 @@ def dense_config(name, s):
                        bos_token_id=1, eos_token_id=(2,))
 
 
-MODELS = {"kesirax": kesirax_config, "mixtral": mixtral_config, "fikizen": fikizen_config, "dense": dense_config}
-PAIRS = (("kesirax", "mixtral"), ("fikizen", "dense"))
+def kemavik_config(name, s):
+    """Four layers: decayed linear attention + dense feed-forward, differential attention + routed experts,
+    differential attention on that layer's keys and values + dense feed-forward, linear attention + dense
+    feed-forward. A differential head = two 64-dim maps over one 128-dim value head; plain causal attention."""
+    from ..config import DenseFFSpec, HybridLayerSpec, KemavikConfig, RoutedMoESpec, WindowAttentionSpec, WkvSpec
+
+    H, kv = s["heads"], max(1, s["heads"] // 4)
+    attn = dict(heads=H, kv_heads=kv, dim=64, vdim=128, scale=64 ** -0.5, bias=True, out_bias=True, head_norm=True,
+                maps=2, diff=0.6)
+    wkv = WkvSpec(heads=s["width"] // 64, dim=64, decay_rank=64)
+    d = DenseFFSpec(s["dense_ff"], "relu2")
+    moe = RoutedMoESpec(experts=s["experts"], top=s["top"], ff=s["ff"], identity=2, scale=1.5, shared_ff=s["ff"])
+    layers = (HybridLayerSpec(wkv, d), HybridLayerSpec(WindowAttentionSpec(**attn), moe),
+              HybridLayerSpec(WindowAttentionSpec(kv_from=1, **attn), d), HybridLayerSpec(wkv, d))
+    return KemavikConfig(name=f"kemavik-{name}", hidden_size=s["width"], vocab_size=s["vocab"], layers=layers,
+                         max_position_embeddings=16384, eos_token_id=(2,), bos_token_id=1)
+
+
+MODELS = {"kesirax": kesirax_config, "mixtral": mixtral_config, "fikizen": fikizen_config, "dense": dense_config,
+          "kemavik": kemavik_config}
+PAIRS = (("kesirax", "mixtral"), ("fikizen", "dense"), ("kemavik", "fikizen"), ("kemavik", "mixtral"))
 
 
 def measure(mcfg, batch, prompt_len, new_tokens, device="cuda", repeats=2):

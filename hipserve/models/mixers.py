@@ -30,8 +30,8 @@ them is one op of the op set:
   recurrence from the sequence's state slot, per-head output norm and SiLU gate) -> output
   projection.
 * routed experts (``RoutedMoE``): 32-bit router logits -> ``route_topk`` (softmax, corrected
-  selection, weights) -> ``moe_align`` tiles -> ``expert_gemm`` (gate | up) -> ``activation``
-  (silu_mul) -> ``expert_gemm`` (down); the weighted combine, the identity experts and the shared
+  selection, weights) -> ``moe_align`` tiles -> ``expert_gemm`` (gate | up, SiLU gate in its epilogue)
+  -> ``expert_gemm`` (down); the weighted combine, the identity experts and the shared
   expert are folded into the residual update (``add_normed``).
 * gated delta rule: merged [q | k | v | beta | decay | gate] projection -> ``gated_delta``
   (causal convolution + SiLU, unit q / k, the recurrence from the sequence's state slot,
@@ -620,12 +620,10 @@ class RoutedMoE:
         tile_expert = torch.empty(cap // tile, dtype=torch.int32, device=dev)
         pair_slot = torch.empty(P, dtype=torch.int32, device=dev)
         ops.moe_align(ids.view(-1), nb, tile, slots, tile_expert, pair_slot)
-        gu = torch.empty(cap, 2 * s.ff, device=dev, dtype=h.dtype)
-        ops.expert_gemm(gu, h, self.w_gu, slots, tile_expert, tile, s.top, False)
         act = torch.empty(cap, s.ff, device=dev, dtype=h.dtype)
-        ops.activation(act, gu, "silu_mul")
+        ops.expert_gemm(act, h, self.w_gu, slots, tile_expert, tile, s.top, 2)      # silu(gate) * up in the epilogue
         ye = torch.empty(cap, self.hidden, device=dev, dtype=h.dtype)
-        ops.expert_gemm(ye, act, self.w_down, slots, tile_expert, tile, 0, False)
+        ops.expert_gemm(ye, act, self.w_down, slots, tile_expert, tile, 0, 0)
         shared = None
         if s.shared_ff:
             g = F.linear(h, self.ws_gu)

