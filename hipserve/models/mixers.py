@@ -582,6 +582,7 @@ class RoutedMoE:
         self.w_gu = None          # [E, 2 * ff, hidden]: gate rows, then up rows
         self.w_down = None        # [E, hidden, ff]
         self.ws_gu = self.ws_down = None   # the shared expert's [2 * shared_ff, hidden], [hidden, shared_ff]
+        self.packed = None        # (gate | up, down) in the packed grouped-GEMM layout, made at the first large batch
 
     def load(self, get, prefix: str):
         s, dt, dev = self.spec, self.dtype, self.device
@@ -614,6 +615,9 @@ class RoutedMoE:
         ops.route_topk(ids, wts, _linear32(h, self.w_router), self.correction, s.top, s.scale, s.experts)
         # the identity experts share one bucket (s.experts) that no GEMM tile serves
         P, nb = T * s.top, s.experts + (1 if s.identity else 0)
+        if self._packed_ok(h, P, nb):
+            ye, pair_slot = self._experts_packed(h, ids, P, nb)
+            return ye, pair_slot, ids, wts, s.experts, h, self._shared(h)
         tile = MOE_TILE_LARGE if P >= 4 * MOE_TILE_LARGE * nb else MOE_TILE
         cap = -(-(P + nb * (tile - 1)) // tile) * tile
         slots = torch.empty(cap, dtype=torch.int32, device=dev)
@@ -624,13 +628,52 @@ class RoutedMoE:
         ops.expert_gemm(act, h, self.w_gu, slots, tile_expert, tile, s.top, 2)      # silu(gate) * up in the epilogue
         ye = torch.empty(cap, self.hidden, device=dev, dtype=h.dtype)
         ops.expert_gemm(ye, act, self.w_down, slots, tile_expert, tile, 0, 0)
-        shared = None
-        if s.shared_ff:
-            g = F.linear(h, self.ws_gu)
-            a = torch.empty(T, s.shared_ff, device=dev, dtype=h.dtype)
-            ops.activation(a, g, "silu_mul")
-            shared = F.linear(a, self.ws_down)
-        return ye, pair_slot, ids, wts, s.experts, h, shared
+        return ye, pair_slot, ids, wts, s.experts, h, self._shared(h)
+
+    def _shared(self, h: torch.Tensor):
+        if not self.spec.shared_ff:
+            return None
+        g = F.linear(h, self.ws_gu)
+        a = torch.empty(h.shape[0], self.spec.shared_ff, device=h.device, dtype=h.dtype)
+        self.ops.activation(a, g, "silu_mul")
+        return F.linear(a, self.ws_down)
+
+    def _packed_ok(self, h: torch.Tensor, P: int, nb: int) -> bool:
+        s = self.spec
+        return (getattr(self.ops, "name", "") == "hip" and h.dtype == torch.bfloat16 and nb <= 128
+                and self.hidden % 256 == 0 and s.ff % 256 == 0
+                and P >= MOE_PACKED_MIN_PAIRS_PER_EXPERT * nb and not torch.cuda.is_current_stream_capturing())
+
+    def _experts_packed(self, h: torch.Tensor, ids: torch.Tensor, P: int, nb: int):
+        """Large bf16 batches: the experts as two launches of the packed-layout grouped GEMM of the dense
+        families' MoE prefill (token rows gathered through the slot table inside the first one, the SiLU gate
+        in its epilogue). The identity bucket sorts last, so the GEMMs simply stop before its tiles."""
+        from ..ops import gemm
+
+        s, dev = self.spec, h.device
+        op = self.ops._op  # the core kernel library
+        E, H, ff = s.experts, self.hidden, s.ff
+        if self.packed is None:
+            pgu = torch.empty(E, 2 * ff * H, dtype=h.dtype, device=dev)
+            pd = torch.empty(E, -(-H // 128) * 128 * ff, dtype=h.dtype, device=dev)
+            op.pack_decode_weight(pgu, self.w_gu, True)
+            op.pack_decode_weight(pd, self.w_down, False)
+            self.packed = (pgu, pd)
+        tile = 128 * gemm.PW_WM
+        cap = -(-(P + nb * (tile - 1)) // tile) * tile
+        slots = torch.empty(cap, dtype=torch.int32, device=dev)
+        tile_expert = torch.empty(cap // tile, dtype=torch.int32, device=dev)
+        ntiles = torch.empty(1, dtype=torch.int32, device=dev)
+        pair_slot = torch.empty(P, dtype=torch.int32, device=dev)
+        op.moe_align(ids.view(-1), nb, tile, slots, tile_expert, ntiles, pair_slot, None)
+        if nb > E:   # tiles of experts with weights
+            ntiles = ((tile_expert >= 0) & (tile_expert < E)).sum(dtype=torch.int32).view(1)
+        pgu, pd = self.packed
+        act = torch.empty(cap, ff, dtype=h.dtype, device=dev)
+        op.prefill_gemm_packed_grouped(act, h, pgu, 2 * ff, 2, tile_expert, ntiles, gemm.PW_WM, gemm.PW_RW, slots, s.top)
+        ye = torch.empty(cap, H, dtype=h.dtype, device=dev)
+        op.prefill_gemm_packed_grouped(ye, act, pd, H, 0, tile_expert, ntiles, gemm.PW_WM, gemm.PW_RW)
+        return ye, pair_slot
 
 
 def make_ff(spec, hidden: int, device, dtype, ops):

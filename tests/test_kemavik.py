@@ -213,6 +213,25 @@ def test_routed_experts_alone(target, shape):
         assert torch.equal(got_ids.sort(-1).values, idx.clamp(max=f["router"]["experts"]).sort(-1).values)
 
 
+@pytest.mark.gpu
+def test_routed_experts_large_batch_gpu():
+    """Enough pairs per expert that the experts run as the packed grouped GEMM of the dense families' prefill
+    (gate in its epilogue, the identity bucket's tiles left out)."""
+    dev, ops = torch.device("cuda"), get_ops("cuda")
+    f = O.moe(experts=2, top=2, ff=256, identity=1, shared=0)
+    cfg = O.make_config([O.wkv_layer(mlp=f)], width=256)
+    W = O.make_weights(cfg, seed=19)
+    h = rows(500, 256, 3)
+    y = O.moe_ff(h.double(), f, d64(W), "l0.mlp.")
+    ff = make_ff(KemavikConfig.from_dict(cfg).layers[0].mlp, 256, dev, torch.bfloat16, ops)
+    ff.load(lambda k: W[k], "l0.mlp.")
+    assert ff._packed_ok(h.to(dev, torch.bfloat16), 1000, 3)
+    res = torch.zeros(500, 256, device=dev)
+    out = torch.empty(500, 256, device=dev, dtype=torch.bfloat16)
+    ops.add_normed(out, res, None, torch.ones(256, device=dev), EPS, ff.forward(h.to(dev, torch.bfloat16)))
+    assert ff.packed is not None and rel_err(res, O.rms(y, EPS)) < 3e-2
+
+
 @pytest.mark.parametrize("target", TARGETS)
 def test_dense_feed_forward_and_output_norm_alone(target):
     dev, dt = torch.device(target[0]), getattr(torch, target[1])
