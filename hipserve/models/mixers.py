@@ -639,8 +639,10 @@ class RoutedMoE:
         return F.linear(a, self.ws_down)
 
     def _packed_ok(self, h: torch.Tensor, P: int, nb: int) -> bool:
+        from ..ops import core_built
+
         s = self.spec
-        return (getattr(self.ops, "name", "") == "hip" and h.dtype == torch.bfloat16 and nb <= 128
+        return (getattr(self.ops, "name", "") == "hip" and h.dtype == torch.bfloat16 and nb <= 128 and core_built()
                 and self.hidden % 256 == 0 and s.ff % 256 == 0
                 and P >= MOE_PACKED_MIN_PAIRS_PER_EXPERT * nb and not torch.cuda.is_current_stream_capturing())
 

@@ -80,6 +80,12 @@ def load_delta_library() -> str:
         return _LIB_DELTA
 
 
+def core_built() -> bool:
+    """True when hipserve/_C.so exists (loaded or not): callers that only PREFER a core kernel ask this, so
+    that a model which can do without never triggers the core library's build."""
+    return _loaded or os.path.exists(_LIB)
+
+
 def native_available() -> bool:
     try:
         load_library()

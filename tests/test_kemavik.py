@@ -389,7 +389,7 @@ def test_far_keys_at_page_borders(tmp_path, target, kv_reader):
 
 
 @pytest.mark.parametrize("target", TARGETS)
-@pytest.mark.parametrize("variant", ["ones", "no_mlp", "readers", "wide", "unequal"])
+@pytest.mark.parametrize("variant", ["ones", "no_mlp", "readers", "wide", "unequal", "odd"])
 def test_other_sizes(tmp_path, target, variant):
     d = O.dense(ff=8)
     if variant == "ones":           # everything 1 that can be
@@ -408,6 +408,10 @@ def test_other_sizes(tmp_path, target, variant):
         layers = [O.attn_layer(heads=2, kv_heads=1, dim=72, vdim=136, mlp=O.dense(ff=70)), O.wkv_layer(heads=2, dim=66),
                   O.attn_layer(heads=2, kv_heads=2, dim=20, vdim=7, mlp=O.moe(experts=3, ff=65, shared=9))]
         cfg = O.make_config(layers, width=24)
+    elif variant == "odd":          # nothing a multiple of 4; experts on a linear-attention layer
+        layers = [O.wkv_layer(heads=3, dim=5, mlp=O.moe(experts=3, top=2, identity=1, ff=7, shared=5)),
+                  O.attn_layer(heads=3, kv_heads=1, dim=6, vdim=5, mlp=O.dense(ff=11)), O.attn_layer(heads=9, kv_heads=1, dim=6, vdim=5, kv_from=1)]
+        cfg = O.make_config(layers, width=30, vocab=53)
     else:                           # heads * vdim, 2 * heads * dim and the width all differ; vdim < dim; group of 3
         layers = [O.attn_layer(heads=6, kv_heads=2, dim=16, vdim=8, mlp=O.moe(experts=6, top=2, identity=0, ff=20, shared=12)),
                   O.wkv_layer(heads=3, dim=16, mlp=O.dense(ff=100))]
