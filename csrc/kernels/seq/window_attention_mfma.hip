@@ -60,7 +60,7 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
     const int* __restrict__ seq_ctx, const int* __restrict__ seq_bt, int bt_width, int seq0, int seq1, int tq, int hc,
     int hchunks, int heads, int kv_heads, int dim, int vdim, int gate_off, float scale, int window, bool sink,
     float out_scale, int part_keys, float* __restrict__ ws_acc, float* __restrict__ ws_ml, int row_base, int ws_rows,
-    float lam, float post, float eps) {
+    float lam, float post, float eps, bool one_row_seqs, bool qvec) {
   static_assert(!DIFF || MT == 2, "the two row tiles of a wave are the two maps");
   constexpr int kLd = KLd<KS>::v;
   constexpr int kMaps = DIFF ? 2 : 1;
@@ -68,7 +68,13 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
   __shared__ __attribute__((aligned(16))) unsigned short kt[kMaps * kKeys * kLd];  // [map][key][dim]
   __shared__ __attribute__((aligned(16))) unsigned short vt[NV * 16 * kVLd];  // [value dim][permuted key]
   int s, tok0;
-  if (!find_tile_rows(seq_cu, seq0, seq1, tq, blockIdx.x, s, tok0)) return;
+  if (one_row_seqs) {  // decode rows: sequence seq0 + x has the one row of workgroup x (no walk over the row counts)
+    s = seq0 + blockIdx.x;
+    tok0 = 0;
+    if (s >= seq1) return;
+  } else if (!find_tile_rows(seq_cu, seq0, seq1, tq, blockIdx.x, s, tok0)) {
+    return;
+  }
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int group = heads / kv_heads;
@@ -104,10 +110,14 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       u16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (qvec) {  // rows and heads start at multiples of 8 elements: one 16-byte load (dim % 8 == 0)
+        if (sact[mt] && 32 * ks + 8 * g < dim) v = *reinterpret_cast<const u16x8*>(src + 32 * ks + 8 * g);
+      } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int d = 32 * ks + 8 * g + e;
-        if (sact[mt] && d < dim) v[e] = src[d];
+        for (int e = 0; e < 8; ++e) {
+          const int d = 32 * ks + 8 * g + e;
+          if (sact[mt] && d < dim) v[e] = src[d];
+        }
       }
       qf[mt][ks] = __builtin_bit_cast(bf16x8, v);
     }
@@ -389,11 +399,14 @@ void launch_mfma(unsigned short* out, long out_ld, const unsigned short* proj, l
   const int hchunks = (group + hc - 1) / hc;
   // split rows (decode): one token per workgroup; else as many consecutive tokens as fit the rows
   const int tq = nparts > 1 ? 1 : rows / hc;
-  dim3 grid(rows_bound / tq + (seq1 - seq0), kv_heads * hchunks, nparts);
+  // split rows are decode rows, one per sequence: workgroup x serves sequence seq0 + x
+  const bool one_row_seqs = nparts > 1 && rows_bound == seq1 - seq0;
+  const bool qvec = proj_ld % 8 == 0 && reinterpret_cast<uintptr_t>(proj) % 16 == 0;
+  dim3 grid(one_row_seqs ? rows_bound : rows_bound / tq + (seq1 - seq0), kv_heads * hchunks, nparts);
   window_attention_mfma_kernel<KS, NV, MT, DIFF><<<grid, kThreads, 0, s>>>(
       out, out_ld, proj, proj_ld, cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1, tq, hc, hchunks,
       heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale, part_keys, ws_acc, ws_ml, row_base,
-      rows_bound, lam, post, eps);
+      rows_bound, lam, post, eps, one_row_seqs, qvec);
   if (nparts > 1 && DIFF)
     window_attention_diff_reduce_kernel<<<dim3(rows_bound, heads), 128, 0, s>>>(
         out, out_ld, ws_acc, ws_ml, proj, proj_ld, gate_off, nparts, heads, rows_bound, row_base, vdim, out_scale, lam,

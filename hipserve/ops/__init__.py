@@ -306,6 +306,8 @@ class KernelOps:
             if nd:
                 span = min(sp.window, meta.max_ctx or sp.window) if sp.window > 0 else meta.max_ctx
                 part = self.WINDOW_DECODE_RUN
+                if span >= 16 * part:   # long runs of keys: fewer, longer runs per row (measured at 2k and 8k keys)
+                    part *= 2
                 while -(-span // part) > 64:
                     part *= 2
                 nparts = max(1, -(-span // part))
