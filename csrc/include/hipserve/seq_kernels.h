@@ -124,6 +124,11 @@ void launch_token_shift(void* out, const float* x, float* state, const float* mu
 void launch_wkv(void* out, float* S, const void* proj, const float* wl, const float* w0, const float* u,
                 const float* norm_w, const int* seq_cu, const int* seq_ctx, const int* seq_state, int nseq, int T,
                 float* scratch, int heads, int dim, float eps, bool f32, hipStream_t s);
+// The same for steps in which every sequence has ONE row, in one launch: low [T, rank] is the decay bottleneck's
+// output BEFORE its tanh, w2 [heads * dim, rank] its up-projection; dim <= 256.
+void launch_wkv_step(void* out, float* S, const void* proj, long T, const void* low, const void* w2, int rank,
+                     const float* w0, const float* u, const float* norm_w, const int* seq_cu, const int* seq_ctx,
+                     const int* seq_state, int nseq, int heads, int dim, float eps, bool f32, hipStream_t s);
 // kind 0: tanh; 1: c0 z^2 + z/2 (z > 0), c1 (exp(z) - 1 - z) + z/2 (z <= 0); 2: max(z, 0)^2;
 // 3: x rows = [gate | up] of `cols` each, out = silu(gate) * up.
 void launch_activation(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, int kind, float c0,

@@ -503,6 +503,66 @@ __global__ __launch_bounds__(NT) void wkv_scan_kernel(
       if (v0 + cv < dim && k0 + i < dim) Sp[(long)(k0 + i) * dim + v0 + cv] = st[cv][i];
 }
 
+// Decode rows (one row per sequence): the whole linear-attention step of one (sequence, head) in one workgroup:
+// decay bottleneck up-projection wl = w2 . tanh(low) (the tanh rounded to the activation type, as the batched path
+// stores it), decay, bonus, read-out from the state before its update, state update, per-head RMS norm, weight and
+// SiLU gate. Thread v owns state column v (dim <= blockDim): it walks the key channels, so state reads and writes
+// are coalesced across the threads.
+template <typename T>
+__global__ __launch_bounds__(256) void wkv_step_kernel(
+    T* __restrict__ out, float* __restrict__ S, const T* __restrict__ proj, long T_, const T* __restrict__ low,
+    const T* __restrict__ w2, int rank, const float* __restrict__ w0, const float* __restrict__ u,
+    const float* __restrict__ norm_w, const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx,
+    const int* __restrict__ seq_state, int heads, int dim, float eps) {
+  extern __shared__ float sm[];   // [rank] tanh(low), then w, k, r [dim] each
+  __shared__ float red[16];
+  float* tl = sm;
+  float* sw = sm + rank;
+  float* sk = sw + dim;
+  float* sr = sk + dim;
+  const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
+  const int t = seq_cu[s];
+  if (seq_cu[s + 1] - t != 1) return;   // sequences without a row in this step
+  const long N = (long)heads * dim;
+  for (int j = tid; j < rank; j += 256) {
+    float v = tanhf(ldf<T>(low, (long)t * rank + j));
+    if constexpr (sizeof(T) == 2) v = bf16_to_f32(f32_to_bf16(v));
+    tl[j] = v;
+  }
+  __syncthreads();
+  float val = 0.f, gate = 0.f, b = 0.f;
+  if (tid < dim) {
+    const long c = (long)h * dim + tid;
+    float a = 0.f;
+    for (int j = 0; j < rank; ++j) a = __builtin_fmaf(ldf<T>(w2, c * rank + j), tl[j], a);
+    const float r = ldf<T>(proj, t * N + c), k = ldf<T>(proj, (T_ + t) * N + c);
+    sw[tid] = expf(-expf(a + w0[c]));
+    sk[tid] = k;
+    sr[tid] = r;
+    val = ldf<T>(proj, (2 * T_ + t) * N + c);
+    gate = ldf<T>(proj, (3 * T_ + t) * N + c);
+    b = r * u[c] * k;
+  }
+  b = block_sum(b, red);   // also orders the writes of sw / sk / sr before the reads below
+  float o = 0.f;
+  if (tid < dim) {
+    float* Sp = S + (((long)seq_state[s] * heads + h) * dim) * dim + tid;
+    const bool carried = seq_ctx[s] - 1 > 0;
+    o = val * b;
+#pragma unroll 8
+    for (int k = 0; k < dim; ++k) {
+      const float st = carried ? Sp[(long)k * dim] : 0.f;
+      o = __builtin_fmaf(st, sr[k], o);
+      Sp[(long)k * dim] = __builtin_fmaf(sw[k], st, sk[k] * val);
+    }
+  }
+  const float ss = block_sum(tid < dim ? o * o : 0.f, red);
+  if (tid < dim) {
+    const long c = (long)h * dim + tid;
+    stf<T>(out, t * N + c, o / sqrtf(ss / (float)dim + eps) * norm_w[c] * gate * sigmoid_f(gate));
+  }
+}
+
 // One wave per (token, head): out = o / rms(o) * w[head * w_stride + e] * act(gate) * scale.
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(
@@ -698,6 +758,22 @@ void launch_wkv(void* out, float* S, const void* proj, const float* wl, const fl
   else
     head_norm_gate<unsigned short>(out, N, o, (const unsigned short*)proj + 3 * (long)T * N, N, 0, norm_w, dim, T, heads,
                                    dim, eps, true, 1.f, s);
+}
+
+void launch_wkv_step(void* out, float* S, const void* proj, long T, const void* low, const void* w2, int rank,
+                     const float* w0, const float* u, const float* norm_w, const int* seq_cu, const int* seq_ctx,
+                     const int* seq_state, int nseq, int heads, int dim, float eps, bool f32, hipStream_t s) {
+  if (nseq <= 0 || T <= 0) return;
+  dim3 grid(heads, nseq);
+  const size_t smem = (size_t)(rank + 3 * dim) * sizeof(float);
+  if (f32)
+    wkv_step_kernel<float><<<grid, 256, smem, s>>>((float*)out, S, (const float*)proj, T, (const float*)low,
+                                                   (const float*)w2, rank, w0, u, norm_w, seq_cu, seq_ctx, seq_state,
+                                                   heads, dim, eps);
+  else
+    wkv_step_kernel<unsigned short><<<grid, 256, smem, s>>>(
+        (unsigned short*)out, S, (const unsigned short*)proj, T, (const unsigned short*)low, (const unsigned short*)w2,
+        rank, w0, u, norm_w, seq_cu, seq_ctx, seq_state, heads, dim, eps);
 }
 
 void launch_activation(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, int kind, float c0,

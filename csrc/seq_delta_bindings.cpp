@@ -295,6 +295,31 @@ void wkv(at::Tensor& out, at::Tensor& S, const at::Tensor& proj, const at::Tenso
                        dim, (float)eps, f32, cur_stream());
 }
 
+void wkv_step(at::Tensor& out, at::Tensor& S, const at::Tensor& proj, const at::Tensor& low, const at::Tensor& w2,
+              const at::Tensor& w0, const at::Tensor& u, const at::Tensor& norm_w, const at::Tensor& seq_cu,
+              const at::Tensor& seq_ctx, const at::Tensor& seq_state, int64_t heads, int64_t dim, double eps) {
+  CHECK_DEV(proj); CHECK_CONTIG(proj); CHECK_CONTIG(out); CHECK_CONTIG(low); CHECK_CONTIG(w2); CHECK_F32(S); CHECK_F32(w0);
+  CHECK_F32(u); CHECK_F32(norm_w); CHECK_I32(seq_cu); CHECK_I32(seq_ctx); CHECK_I32(seq_state);
+  const bool f32 = is_f32(proj, "wkv_step");
+  TORCH_CHECK(out.scalar_type() == proj.scalar_type() && low.scalar_type() == proj.scalar_type() &&
+              w2.scalar_type() == proj.scalar_type());
+  TORCH_CHECK(heads >= 1 && dim >= 1 && dim <= 256, "wkv_step: sizes");
+  const long N = heads * dim, nseq = seq_ctx.numel();
+  TORCH_CHECK(proj.dim() == 3 && proj.size(0) == 4 && proj.size(2) == N);
+  const long T = proj.size(1);
+  TORCH_CHECK(low.dim() == 2 && low.size(0) == T && w2.dim() == 2 && w2.size(0) == N && w2.size(1) == low.size(1));
+  const long rank = low.size(1);
+  TORCH_CHECK((rank + 3 * dim) * 4 <= 60 * 1024, "wkv_step: bottleneck too wide");
+  TORCH_CHECK(out.numel() == T * N && w0.numel() == N && u.numel() == N && norm_w.numel() == N);
+  TORCH_CHECK(S.dim() == 4 && S.size(1) == heads && S.size(2) == dim && S.size(3) == dim);
+  TORCH_CHECK(seq_cu.numel() == nseq + 1 && seq_state.numel() >= nseq && nseq <= 65535);
+  c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
+  hipserve::launch_wkv_step(out.data_ptr(), S.data_ptr<float>(), proj.data_ptr(), T, low.data_ptr(), w2.data_ptr(), rank,
+                            w0.data_ptr<float>(), u.data_ptr<float>(), norm_w.data_ptr<float>(),
+                            seq_cu.data_ptr<int>(), seq_ctx.data_ptr<int>(), seq_state.data_ptr<int>(), nseq, heads,
+                            dim, (float)eps, f32, cur_stream());
+}
+
 void route_topk(at::Tensor& ids, at::Tensor& wts, const at::Tensor& logits, const at::Tensor& correction, int64_t top,
                 double scale, int64_t E) {
   CHECK_DEV(logits); CHECK_F32(logits); CHECK_F32(correction); CHECK_F32(wts); CHECK_I32(ids);
@@ -339,6 +364,8 @@ TORCH_LIBRARY(hipserve_delta, m) {
         "Tensor seq_state) -> ()");
   m.def("wkv(Tensor(a!) out, Tensor(b!) S, Tensor proj, Tensor wl, Tensor w0, Tensor u, Tensor norm_w, Tensor seq_cu, "
         "Tensor seq_ctx, Tensor seq_state, Tensor(c!) scratch, int heads, int dim, float eps) -> ()");
+  m.def("wkv_step(Tensor(a!) out, Tensor(b!) S, Tensor proj, Tensor low, Tensor w2, Tensor w0, Tensor u, Tensor norm_w, "
+        "Tensor seq_cu, Tensor seq_ctx, Tensor seq_state, int heads, int dim, float eps) -> ()");
   m.def("route_topk(Tensor(a!) ids, Tensor(b!) wts, Tensor logits, Tensor correction, int top, float scale, int E) -> ()");
   m.def("moe_align(Tensor ids, int E, int tile, Tensor(a!) slots, Tensor(b!) tile_expert, Tensor(c!) pair_slot) -> ()");
   m.def("expert_gemm(Tensor(a!) out, Tensor x, Tensor w, Tensor slots, Tensor tile_expert, int tile, int gather_k, "
@@ -356,6 +383,7 @@ TORCH_LIBRARY_IMPL(hipserve_delta, CUDA, m) {
   m.impl("add_normed", &add_normed);
   m.impl("token_shift", &token_shift);
   m.impl("wkv", &wkv);
+  m.impl("wkv_step", &wkv_step);
   m.impl("route_topk", &route_topk);
   m.impl("moe_align", &moe_align);
   m.impl("expert_gemm", &expert_gemm);

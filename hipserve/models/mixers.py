@@ -351,6 +351,7 @@ class Wkv:
     cache_dim = 0
     input32 = True      # forward reads the 32-bit stream itself, not its rounding to the activation type
     BLENDS = ("r", "k", "v", "g", "w")
+    STEP_MAX_DIM, STEP_MAX_RANK = 256, 4096   # sizes the one-row-per-sequence kernel takes
 
     def __init__(self, spec: WkvSpec, hidden: int, eps: float, device, dtype, ops):
         self.spec, self.hidden, self.eps, self.device, self.dtype, self.ops = spec, hidden, eps, device, dtype, ops
@@ -397,9 +398,13 @@ class Wkv:
         ops.token_shift(mixed, x, state[1], self.mu, meta)
         proj = torch.bmm(mixed[:4], self.w_in_t)                       # [4, T, heads * dim]: r, k, v, gate
         low = F.linear(mixed[4], self.w1)
+        out = torch.empty(T, s.size, device=x.device, dtype=self.dtype)
+        if meta.max_q == 1 and s.dim <= self.STEP_MAX_DIM and low.shape[1] <= self.STEP_MAX_RANK:
+            # every sequence brings one row (decode steps): bottleneck, recurrence, norm and gate in one launch
+            ops.wkv_step(out, state[0], proj, low, self.w2, self.w0, self.u, self.norm, s, self.eps, meta)
+            return F.linear(out, self.w_o)
         ops.activation(low, low, "tanh")
         wl = _linear32(low, self.w2)
-        out = torch.empty(T, s.size, device=x.device, dtype=self.dtype)
         ops.wkv(out, state[0], proj, wl, self.w0, self.u, self.norm, s, self.eps, meta)
         return F.linear(out, self.w_o)
 

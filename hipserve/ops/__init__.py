@@ -358,6 +358,12 @@ class KernelOps:
         self._delta.wkv(out, state, proj, wl, w0, u, norm_w, meta.seq_cu, meta.seq_ctx, meta.seq_state, scratch,
                         sp.heads, sp.dim, eps)
 
+    def wkv_step(self, out, state, proj, low, w2, w0, u, norm_w, sp, eps, meta):
+        """``wkv`` for steps in which every sequence has one row (``meta.max_q`` == 1), the decay bottleneck's
+        tanh and up-projection included (``low``: its output before the tanh): one launch."""
+        self._delta.wkv_step(out, state, proj, low, w2, w0, u, norm_w, meta.seq_cu, meta.seq_ctx, meta.seq_state,
+                             sp.heads, sp.dim, eps)
+
     ROUTER_MAX_OUTPUTS = 256
 
     def route_topk(self, ids, wts, logits, correction, top, scale, E):
@@ -520,6 +526,11 @@ class ReferenceOps:
         ref.token_shift(out, x, state, mu, meta.seq_cu, meta.seq_ctx, meta.seq_state)
 
     def wkv(self, out, state, proj, wl, w0, u, norm_w, sp, eps, meta):
+        ref.wkv(out, state, proj, wl, w0, u, norm_w, sp, eps, meta.seq_cu, meta.seq_ctx, meta.seq_state)
+
+    def wkv_step(self, out, state, proj, low, w2, w0, u, norm_w, sp, eps, meta):
+        t = torch.tanh(low.float()).to(low.dtype)
+        wl = torch.nn.functional.linear(t.float(), w2.float())
         ref.wkv(out, state, proj, wl, w0, u, norm_w, sp, eps, meta.seq_cu, meta.seq_ctx, meta.seq_state)
 
     def route_topk(self, ids, wts, logits, correction, top, scale, E):
