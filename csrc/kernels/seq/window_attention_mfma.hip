@@ -61,7 +61,8 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
     int hchunks, int heads, int kv_heads, int dim, int vdim, int gate_off, float scale, int window, bool sink,
     float out_scale, int part_keys, float* __restrict__ ws_acc, float* __restrict__ ws_ml, int row_base, int ws_rows,
     float lam, float post, float eps, bool one_row_seqs, bool qvec) {
-  static_assert(!DIFF || MT == 2, "the two row tiles of a wave are the two maps");
+  static_assert(!DIFF || MT % 2 == 0, "a wave's row tiles come in pairs: the two maps of the same 16 rows");
+  constexpr int RT = DIFF ? MT / 2 : MT;   // distinct 16-row tiles per wave; tile mt is rows mt / kMaps, map mt % kMaps
   constexpr int kLd = KLd<KS>::v;
   constexpr int kMaps = DIFF ? 2 : 1;
   constexpr int kKF = (kMaps * KS * 4 + kFT - 1) / kFT, kVF = (NV * 2 + kFT - 1) / kFT;  // 16-byte chunks per thread and tile
@@ -99,14 +100,14 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
   float m_run[MT], l_run[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int sr = DIFF ? 16 * wave + c : 16 * (wave * MT + mt) + c;
+    const int sr = 16 * (wave * RT + (DIFF ? mt >> 1 : mt)) + c;
     const int srt = sr / hc, srh = sr % hc;
     sact[mt] = srt < ntok && srh < nh;
     head[mt] = kvh * group + h0 + (sact[mt] ? srh : 0);
     trow[mt] = r0 + tok0 + (sact[mt] ? srt : 0);
     spos[mt] = p_first + srt;
     s_lo[mt] = window > 0 ? max(0, spos[mt] - window + 1) : 0;
-    const unsigned short* src = proj + trow[mt] * proj_ld + ((long)head[mt] * kMaps + (DIFF ? mt : 0)) * dim;
+    const unsigned short* src = proj + trow[mt] * proj_ld + ((long)head[mt] * kMaps + (DIFF ? mt & 1 : 0)) * dim;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       u16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -178,10 +179,12 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
       for (int nt = 0; nt < 2; ++nt) {
         if constexpr (DIFF) {
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {  // map mt: its own key tile
+          for (int mp = 0; mp < 2; ++mp) {  // map mp: its own key tile, shared by the wave's row tiles
             const bf16x8 a = __builtin_bit_cast(
-                bf16x8, *reinterpret_cast<const u16x8*>(kt + mt * kKeys * kLd + (16 * nt + c) * kLd + 32 * ks + 8 * g));
-            sc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[mt][ks], sc[mt][nt], 0, 0, 0);
+                bf16x8, *reinterpret_cast<const u16x8*>(kt + mp * kKeys * kLd + (16 * nt + c) * kLd + 32 * ks + 8 * g));
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              sc[2 * rt + mp][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[2 * rt + mp][ks], sc[2 * rt + mp][nt], 0, 0, 0);
           }
         } else {
           const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8*>(kt + (16 * nt + c) * kLd + 32 * ks + 8 * g));
@@ -247,43 +250,47 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
   }
   // lane (c, g) holds value dims 16 j + 4 g .. + 3 of its rows
   if constexpr (DIFF) {
-    if (!sact[0]) return;
-    if (gridDim.z > 1) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {  // the runs of map mt live under "head" 2 head + mt
-        const long wrow = ((long)blockIdx.z * heads * 2 + head[0] * 2 + mt) * ws_rows + (trow[0] - row_base);
-        if (g == 0) { ws_ml[2 * wrow] = m_run[mt]; ws_ml[2 * wrow + 1] = l_run[mt]; }
+    for (int rt = 0; rt < RT; ++rt) {
+      const int m0 = 2 * rt, m1 = 2 * rt + 1;   // the two maps of row tile rt
+      if (!sact[m0]) continue;
+      if (gridDim.z > 1) {
 #pragma unroll
-        for (int j = 0; j < NV; ++j) {
-          const int d = 16 * j + 4 * g;
-          if (d < vdim) *reinterpret_cast<f32x4*>(ws_acc + wrow * vdim + d) = acc[mt][j];
+        for (int mp = 0; mp < 2; ++mp) {  // the runs of map mp live under "head" 2 head + mp
+          const long wrow = ((long)blockIdx.z * heads * 2 + head[m0] * 2 + mp) * ws_rows + (trow[m0] - row_base);
+          if (g == 0) { ws_ml[2 * wrow] = m_run[m0 + mp]; ws_ml[2 * wrow + 1] = l_run[m0 + mp]; }
+#pragma unroll
+          for (int j = 0; j < NV; ++j) {
+            const int d = 16 * j + 4 * g;
+            if (d < vdim) *reinterpret_cast<f32x4*>(ws_acc + wrow * vdim + d) = acc[m0 + mp][j];
+          }
         }
+        continue;
       }
-      return;
-    }
-    const float i0 = l_run[0] > 0.f ? 1.f / l_run[0] : 0.f, i1 = l_run[1] > 0.f ? lam / l_run[1] : 0.f;
-    float ss = 0.f;
+      const float i0 = l_run[m0] > 0.f ? 1.f / l_run[m0] : 0.f, i1 = l_run[m1] > 0.f ? lam / l_run[m1] : 0.f;
+      float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < NV; ++j)
+      for (int j = 0; j < NV; ++j)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float o = acc[0][j][e] * i0 - acc[1][j][e] * i1;  // dims past vdim are zero (zero value rows)
-        acc[0][j][e] = o;
-        ss += o * o;
+        for (int e = 0; e < 4; ++e) {
+          const float o = acc[m0][j][e] * i0 - acc[m1][j][e] * i1;  // dims past vdim are zero (zero value rows)
+          acc[m0][j][e] = o;
+          ss += o * o;
+        }
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      float f = out_scale * post / sqrtf(ss / (float)vdim + eps);
+      if (gate_off >= 0) f *= sigmoid_f(bf16_to_f32(proj[trow[m0] * proj_ld + gate_off + head[m0]]));
+      unsigned short* dst = out + trow[m0] * out_ld + (long)head[m0] * vdim;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int d = 16 * j + 4 * g;
+        if (d >= vdim) continue;
+        u16x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16(acc[m0][j][e] * f);
+        *reinterpret_cast<u16x4*>(dst + d) = o;
       }
-    ss += __shfl_xor(ss, 16, 64);
-    ss += __shfl_xor(ss, 32, 64);
-    float f = out_scale * post / sqrtf(ss / (float)vdim + eps);
-    if (gate_off >= 0) f *= sigmoid_f(bf16_to_f32(proj[trow[0] * proj_ld + gate_off + head[0]]));
-    unsigned short* dst = out + trow[0] * out_ld + (long)head[0] * vdim;
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const int d = 16 * j + 4 * g;
-      if (d >= vdim) continue;
-      u16x4 o;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16(acc[0][j][e] * f);
-      *reinterpret_cast<u16x4*>(dst + d) = o;
     }
     return;
   }
@@ -394,7 +401,7 @@ void launch_mfma(unsigned short* out, long out_ld, const unsigned short* proj, l
                  int window, bool sink, float out_scale, int nparts, int part_keys, float* ws_acc, float* ws_ml,
                  int row_base, float lam, float post, float eps, hipStream_t s) {
   const int group = heads / kv_heads;
-  const int rows = DIFF ? kRows : kRows * MT;
+  const int rows = kRows * (DIFF ? MT / 2 : MT);
   const int hc = min(group, rows);
   const int hchunks = (group + hc - 1) / hc;
   // split rows (decode): one token per workgroup; else as many consecutive tokens as fit the rows
@@ -439,12 +446,15 @@ void launch_window_attention_mfma(void* out, long out_ld, const void* proj, long
                                 out_scale, nparts, part_keys, ws_acc, ws_ml, row_base, lam, post, eps, s)
   // two row tiles per wave where a prompt portion brings enough rows and the accumulators fit the registers
   const int ks = (dim + 31) / 32, nv = (vdim + 15) / 16;
+  const bool wide = nparts == 1 && (long)rows_bound * (heads / kv_heads) >= 128 * (long)(seq1 - seq0);
   if (maps == 2) {
+    // row tiles come in pairs (the two maps): 64 rows per workgroup. Four tiles per wave (128 rows) measured
+    // slower on 4 x 2048-row prompts (532 against 396 us with 64-dim maps and 128-dim values): too many registers.
     if (ks <= 2 && nv <= 4) HS_WA(2, 4, 2, true);
+    else if (ks <= 2) HS_WA(2, 8, 2, true);   // 64-dim maps over 128-dim values: no score products on padding
     else HS_WA(4, 8, 2, true);
     return;
   }
-  const bool wide = nparts == 1 && (long)rows_bound * (heads / kv_heads) >= 128 * (long)(seq1 - seq0);
   if (ks <= 2 && nv <= 4) { if (wide) HS_WA(2, 4, 2, false); else HS_WA(2, 4, 1, false); }
   else if (ks <= 4 && nv <= 8) { if (wide) HS_WA(4, 8, 2, false); else HS_WA(4, 8, 1, false); }
   else HS_WA(8, 16, 1, false);
