@@ -116,6 +116,28 @@ def test_differential_attention_alone(target, shape):
 
 
 @pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("shape", [dict(heads=4, kv_heads=2, dim=64, vdim=128), dict(heads=2, kv_heads=1, dim=128, vdim=96),
+                                   dict(heads=8, kv_heads=1, dim=32, vdim=64), dict(heads=2, kv_heads=2, dim=16, vdim=256)])
+def test_differential_attention_head_sizes_of_real_models(target, shape):
+    """Head sizes that are multiples of 8 (in bf16 every instantiation of the matrix-core kernel, and the generic
+    kernel for the 256-wide values), with enough keys that rows decoded alone split their keys into several runs."""
+    l = O.attn_layer(**shape)
+    W = O.make_weights(O.make_config([l], width=24), seed=20)
+    h = rows(300, 24, 8).double()
+    want, _ = O.diff_attention_mixer(h, l["mixer"], d64(W), "l0.mix.", EPS)
+    cuts = [(0, 150), (150, 297), (297, 298), (298, 299), (299, 300)]
+    (mix,), dev, dt = build_mixers([l], W, target, 24)
+    meta0, _ = one_seq_meta(1, dev, total=304)
+    cache = torch.zeros(304 // 4 + 3, 4, mix.cache_dim, device=dev, dtype=dt)
+    got = []
+    for a, b in cuts:
+        meta, _ = one_seq_meta(b - a, dev, start=a, total=304)
+        meta.max_ctx = b
+        got.append(mix.forward(h[a:b].to(dev, dt), meta, cache, None))
+    assert rel_err(torch.cat(got), want) < TOL[target[1]]
+
+
+@pytest.mark.parametrize("target", TARGETS)
 def test_second_map_norms_and_biases_matter(target):
     l = O.attn_layer()
     W = O.make_weights(O.make_config([l], width=24), seed=6)
