@@ -562,7 +562,10 @@ class LatentAttentionSpec:
     """Attention through low-rank latents: queries go through a ``q_rank`` latent, keys
     and values are expanded per head from one ``kv_rank`` latent per token, and a
     ``rot_dim`` rotary key part is shared by all heads. Only the latent and the rotary
-    key part are cached. ``window`` 0 = plain causal attention."""
+    key part are cached. ``window`` 0 = plain causal attention. ``interleaved``: the rotation
+    pairs coordinate 2i with 2i + 1 (else i with i + rot_dims / 2). ``gate``: ``head`` multiplies
+    head h's output by sigmoid of one number per head, ``channel`` multiplies the concatenated
+    heads element by element by sigmoid of a projection of that size, ``none`` has no gate."""
     heads: int
     dim: int            # unrotated query/key dims per head
     rot_dim: int        # rotated query/key dims per head (one shared key part)
@@ -573,6 +576,8 @@ class LatentAttentionSpec:
     window: int = 0
     rot_base: float = 10000.0
     rot_dims: int = 0   # leading dims of the rotated part that are rotated (0 = all of rot_dim)
+    interleaved: bool = False
+    gate: str = "head"
 
     kind = "latent_attention"
 
@@ -580,6 +585,11 @@ class LatentAttentionSpec:
     def key_dim(self) -> int:
         """Cached elements per token."""
         return self.kv_rank + self.rot_dim
+
+    @property
+    def gate_size(self) -> int:
+        """Rows of the gate projection."""
+        return {"head": self.heads, "channel": self.heads * self.vdim, "none": 0}[self.gate]
 
 
 @dataclass(frozen=True)
@@ -606,7 +616,10 @@ class WindowAttentionSpec:
     """Grouped-query attention over a sliding window (``window`` keys: the token itself and
     the ``window - 1`` before it; 0 = plain causal) with rotate-half rotary positions on the
     first ``rot_dims`` dims of every head. Options, each independent of the others:
-    ``sink`` adds one to the softmax denominator (a key of score 0 without a value),
+    ``sink`` adds one to the softmax denominator (a key of score 0 without a value), with
+    ``sink_weights`` exp of a learned number per head instead of one,
+    ``softcap`` > 0 passes the scaled scores through ``softcap * tanh(. / softcap)``,
+    ``keep_first`` > 0 keeps the sequence's first ``keep_first`` tokens visible behind the window,
     ``gate`` multiplies head h's output by sigmoid of a per-head projection of the mixer input,
     ``bias`` adds biases in the q / k / v projections, ``qk_norm`` applies a weighted RMS norm
     over the WHOLE q (and k) projection before the rotation, ``head_norm`` one over every
@@ -637,6 +650,9 @@ class WindowAttentionSpec:
     maps: int = 1
     diff: float = 0.0
     kv_from: int | None = None
+    softcap: float = 0.0
+    keep_first: int = 0
+    sink_weights: bool = False
 
     kind = "attention"
 
@@ -716,6 +732,26 @@ class DeltaRuleSpec:
 
 
 @dataclass(frozen=True)
+class MLstmSpec:
+    """Matrix memory (mLSTM): per head a ``dim x vdim`` state S and a normaliser n of ``dim``
+    elements, written with an exponential input gate and decayed by a sigmoid forget gate, both
+    one number per head and token and both capped, ``cap * tanh(. / cap)``, before their
+    non-linearity; a running maximum m of the log gates keeps the exponentials bounded. The
+    read-out ``S^T q / (max(|n . q|, exp(-m)) + 1e-6)`` is divided by its per-head root mean
+    square, weighted and gated by a sigmoid of a projection of the input."""
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+    kind = "mlstm"
+
+    @property
+    def out_size(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclass(frozen=True)
 class ParallelMixerSpec:
     """Two mixers on the same input, their outputs summed with fixed weights."""
     left: object
@@ -728,7 +764,9 @@ class ParallelMixerSpec:
 
 @dataclass(frozen=True)
 class DenseFFSpec:
-    """down(act(up(x))) with one of the op set's elementwise activations (``xielu``, ``relu2``)."""
+    """down(act(up(x))) with one of the op set's elementwise activations (``xielu``, ``relu2``) or
+    ``polynorm``: a N(z) + b N(z^2) + c N(z^3) + e with four learned numbers, N dividing a token's
+    vector by its root mean square."""
     ff: int
     act: str = "xielu"
 
@@ -741,13 +779,19 @@ class RoutedMoESpec:
     the largest score + correction are chosen, weighted by their (uncorrected, not
     renormalised) score times ``scale``. The last ``identity`` router outputs are experts
     without weights that return their input; ``shared_ff`` > 0 adds a gated feed-forward that
-    every token runs."""
+    every token runs. ``groups`` > 1: the router outputs form that many equal groups of
+    neighbours, a group scores the largest corrected score in it, and only the experts of the
+    ``keep_groups`` best groups can be chosen. ``renorm``: the chosen scores are divided by
+    their sum before the scaling."""
     experts: int
     top: int
     ff: int
     identity: int = 0
     scale: float = 1.0
     shared_ff: int = 0
+    groups: int = 1
+    keep_groups: int = 1
+    renorm: bool = False
 
     kind = "routed_moe"
 
@@ -1031,6 +1075,115 @@ class KemavikConfig:
             norm_eps=float(norm.get("eps", 1e-6)), bos_token_id=d.get("bos_token_id"), eos_token_id=eos)
 
 
+@dataclass(frozen=True)
+class TopezenConfig:
+    """Topezen: a decoder given as a list of layers, each a parallel block with two norms,
+
+        x <- x + sigmoid(rg1(norm1 x)) * mixer(norm1 x) + sigmoid(rg2(norm2 x)) * ff(norm2 x)
+
+    where the RMS norms have ONE weight each and ``rg`` are full-width projections with a bias
+    (a gate per channel on each sublayer's result). Mixers: causal latent attention with an
+    interleaved rotation and a per-channel output gate, an mLSTM matrix memory, or grouped-query
+    attention without positions (per-head query / key norms, capped scores, a sliding window that
+    keeps the first tokens, a learned softmax sink per head). Feed-forwards: dense with a
+    PolyNorm activation, or a routed mixture of gated experts (corrected, group-limited top-k
+    selection, renormalised weights, a shared expert); a layer may have none. The embedding is
+    scaled by ``embed_scale``."""
+    name: str = "topezen"
+    architecture: str = "topezen"
+    family: str = "topezen"
+    hidden_size: int = 256
+    vocab_size: int = 512
+    layers: tuple = ()
+    norm_eps: float = 1e-6
+    embed_scale: float = 1.0
+    max_position_embeddings: int = 1 << 20   # rotary angles are computed, not tabulated
+    default_model_len: int = 32768
+    bos_token_id: int | None = None
+    eos_token_id: tuple = ()
+    vision: object = None
+    num_experts: int = 0                      # engine start-up tuning of the dense families keys on it
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def runs(self) -> list:
+        """Layer runs in execution order: (layer index, 0, False); every layer runs once."""
+        return [(i, 0, False) for i in range(len(self.layers))]
+
+    def num_params(self) -> int:
+        H, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size
+        for l in self.layers:
+            m, f = l.mixer, l.mlp
+            n += H * H
+            if isinstance(m, LatentAttentionSpec):
+                n += H * (m.q_rank + m.key_dim + m.gate_size) + m.q_rank * m.heads * (m.dim + m.rot_dim)
+                n += m.kv_rank * m.heads * (m.dim + m.vdim) + m.heads * m.vdim * H
+            elif isinstance(m, MLstmSpec):
+                n += H * (2 * m.heads * m.dim + 3 * m.out_size + 2 * m.heads)
+            else:
+                n += H * (m.q_size + m.cache_dim) + m.heads * m.vdim * H
+            if f is not None:
+                n += H * H
+            if isinstance(f, DenseFFSpec):
+                n += 2 * f.ff * H
+            elif f is not None:
+                n += 3 * H * (f.experts * f.ff + f.shared_ff) + H * f.experts
+        return n
+
+    def replace(self, **kw) -> "TopezenConfig":
+        return dataclasses.replace(self, **kw)
+
+    @staticmethod
+    def from_dict(d: dict, name: str = "model") -> "TopezenConfig":
+        layers = []
+        for l in d["layers"]:
+            m, kind = l["mixer"], l["type"]
+            if kind == "latent_attention":
+                rot = m.get("rot") or {}
+                mixer = LatentAttentionSpec(
+                    heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+                    q_rank=int(m["q_rank"]), kv_rank=int(m["kv_rank"]), scale=float(m["scale"]),
+                    rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims") or m["rot_dim"]),
+                    interleaved=True, gate="channel")
+            elif kind == "mlstm":
+                mixer = MLstmSpec(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                  gate_cap=float(m["gate_cap"]))
+            elif kind == "attention":
+                mask = m.get("mask") or {}
+                mixer = WindowAttentionSpec(
+                    heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                    scale=float(m["scale"]), window=int(mask.get("size") or 0), keep_first=int(mask.get("keep_first") or 0),
+                    softcap=float(m.get("softcap") or 0.0), head_norm=True, sink=True, sink_weights=True)
+            else:
+                raise NotImplementedError(f"unknown mixer {kind!r}")
+            f = l.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind") == "dense":
+                    mlp = DenseFFSpec(ff=int(f["ff"]), act="polynorm")
+                elif f.get("kind") == "moe":
+                    r = f["router"]
+                    g = r.get("groups") or {}
+                    count = int(g.get("count") or 1)
+                    if int(r["experts"]) % count:
+                        raise ValueError("the experts do not divide into equal groups")
+                    mlp = RoutedMoESpec(experts=int(r["experts"]), top=int(r["top"]), ff=int(f["expert"]["ff"]),
+                                        shared_ff=int((f.get("shared") or {}).get("ff") or 0), groups=count,
+                                        keep_groups=int(g.get("keep") or count), renorm=True)
+                else:
+                    raise NotImplementedError(f"unknown feed-forward {f.get('kind')!r}")
+            layers.append(HybridLayerSpec(mixer, mlp))
+        norm = d.get("norm") or {}
+        eos = d.get("eos_token_id", ())
+        eos = tuple(eos) if isinstance(eos, (list, tuple)) else (eos,)
+        return TopezenConfig(
+            name=name, hidden_size=int(d["width"]), vocab_size=int(d["vocab"]), layers=tuple(layers),
+            norm_eps=float(norm.get("eps", 1e-6)), embed_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
+            bos_token_id=d.get("bos_token_id"), eos_token_id=eos)
+
+
 def check_kv_sources(layers):
     """A layer that reads another layer's keys and values must name an earlier attention layer
     with a cache of its own and the same key / value head layout."""
@@ -1055,6 +1208,8 @@ def config_from_dict(d: dict, name: str = "model"):
         return FikizenConfig.from_dict(d, name=name)
     if arch == "kemavik":
         return KemavikConfig.from_dict(d, name=name)
+    if arch == "topezen":
+        return TopezenConfig.from_dict(d, name=name)
     return ModelConfig.from_hf_dict(d, name=name)
 
 

@@ -19,7 +19,8 @@ from .mixers import make_ff, make_mixer
 
 class _Layer:
     def __init__(self):
-        self.norm1 = self.norm2 = None   # [hidden] fp32
+        self.norm1 = self.norm2 = None   # [hidden] fp32 (one number each in designs with single-weight norms)
+        self.b1 = self.b2 = None         # [hidden] fp32: biases of the gates on the sublayers' results, where a design has them
         self.mixer = None
         self.mlp = None
 
@@ -53,7 +54,7 @@ class LayerListModel:
             lw = _Layer()
             lw.mixer = make_mixer(spec.mixer, H, cfg.norm_eps, self.device, dtype, ops)
             if spec.mlp is not None:
-                lw.mlp = make_ff(spec.mlp, H, self.device, dtype, ops)
+                lw.mlp = make_ff(spec.mlp, H, self.device, dtype, ops, cfg.norm_eps)
             self.layers.append(lw)
         self.embed = self.final_norm = self.lm_head = None
         self.capture = None  # a list: the residual stream after every layer run is appended (debugging)

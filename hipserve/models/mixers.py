@@ -43,16 +43,25 @@ them is one op of the op set:
   buffer, and ONE output projection over the concatenated weights sums them.
 * dense feed-forward: up projection -> ``activation`` -> down projection.
 
+* matrix memory (``MLstm``): merged [q | k | v | gate] projection and a 32-bit [input gate | forget
+  gate] projection -> ``mlstm`` (capped log gates, running maximum, the recurrence of the matrix
+  state and its normaliser from the sequence's state slot, read-out, per-head output norm, weight
+  and sigmoid gate) -> output projection.
+
 A mixer's ``forward(h, meta, cache, state)`` gets the layer run's paged cache and state
 tensors (None where it has none); ``cache_dim`` / ``state_shapes`` say what a run needs.
+
+Side projection: a model whose block needs one more projection of a sublayer's input (a gate on
+the sublayer's result, say) attaches its rows to the sublayer's merged input GEMM with
+``attach_side``; after ``forward`` the sublayer's ``side_out`` holds those columns.
 """
 from __future__ import annotations
 
 import torch
 import torch.nn.functional as F
 
-from ..config import (DeltaRuleSpec, DenseFFSpec, GatedDeltaSpec, LatentAttentionSpec, MinGRUSpec, ParallelMixerSpec,
-                      RoutedMoESpec, TableMoESpec, WindowAttentionSpec, WkvSpec)
+from ..config import (DeltaRuleSpec, DenseFFSpec, GatedDeltaSpec, LatentAttentionSpec, MinGRUSpec, MLstmSpec,
+                      ParallelMixerSpec, RoutedMoESpec, TableMoESpec, WindowAttentionSpec, WkvSpec)
 
 MOE_TILE = 32        # slots per expert tile of the expert GEMMs ...
 MOE_TILE_LARGE = 64  # ... when every expert has several tiles' worth of rows on average
@@ -60,6 +69,29 @@ MOE_TILE_LARGE = 64  # ... when every expert has several tiles' worth of rows on
 # GEMM of the dense families' MoE prefill (prefill_gemm_packed.hip: 128-row tiles, X through LDS, the
 # weights pre-shuffled into MFMA operand order) with the squared ReLU in its epilogue
 MOE_PACKED_MIN_PAIRS_PER_EXPERT = 256
+
+
+def attach_side(sub, w: torch.Tensor):
+    """Append the rows of ``w`` [n, hidden] to the merged input projection of a mixer or feed-forward."""
+    name = sub.side_weight
+    cur = getattr(sub, name)
+    w = w.to(sub.device, sub.dtype)
+    setattr(sub, name, w.contiguous() if cur is None else torch.cat([cur, w], 0).contiguous())
+    if getattr(sub, "b_in", None) is not None:
+        sub.b_in = torch.cat([sub.b_in, torch.zeros(w.shape[0], device=sub.device, dtype=sub.b_in.dtype)]).contiguous()
+    sub.side_rows = w.shape[0]
+
+
+def _side(sub, proj: torch.Tensor):
+    n = sub.side_rows
+    sub.side_out = proj[:, proj.shape[1] - n:] if n else None
+
+
+def _deinterleave(w: torch.Tensor, dims: int) -> torch.Tensor:
+    """Rows [..., r, in] of a projection whose outputs are rotated in pairs (2i, 2i + 1): the first ``dims`` rows
+    reordered to [even | odd], so that the rotate-half kernels (pairs i, i + dims / 2) compute the same scores."""
+    idx = torch.cat([torch.arange(0, dims, 2), torch.arange(1, dims, 2), torch.arange(dims, w.shape[-2])])
+    return w.index_select(-2, idx)
 
 
 def _mm32(x: torch.Tensor, w_t: torch.Tensor) -> torch.Tensor:
@@ -72,10 +104,15 @@ def _mm32(x: torch.Tensor, w_t: torch.Tensor) -> torch.Tensor:
 
 
 class LatentAttention:
+    side_weight, side_rows, side_out = "w_in", 0, None
+    state_shapes = None
+    cache_dim = property(lambda self: self.spec.key_dim)
+
     def __init__(self, spec: LatentAttentionSpec, hidden: int, eps: float, device, dtype, ops):
         self.spec, self.hidden, self.eps, self.device, self.dtype, self.ops = spec, hidden, eps, device, dtype, ops
         s = spec
-        self.w_in = None       # [q_rank + kv_rank + rot_dim + heads, hidden]
+        assert s.gate in ("head", "channel", "none")
+        self.w_in = None       # [q_rank + kv_rank + rot_dim + gate rows, hidden]
         self.q_norm = None     # [q_rank] fp32
         self.kv_norm = None    # [kv_rank] fp32
         self.w_uq = None       # [heads * (dim + rot_dim), q_rank]
@@ -90,10 +127,19 @@ class LatentAttention:
 
     def load(self, get, prefix: str):
         s, dt, dev = self.spec, self.dtype, self.device
-        self.w_in = torch.cat([get(prefix + "dq"), get(prefix + "dkv"), get(prefix + "g")], 0).to(dev, dt).contiguous()
+        dkv, uq = get(prefix + "dkv"), get(prefix + "uq")
+        if s.interleaved:
+            # the same permutation of the rotary key rows and of every head's rotary query rows leaves the
+            # scores unchanged and turns the pairs (2i, 2i + 1) into the pairs (i, i + dims / 2) of the kernels
+            rd = s.rot_dims or s.rot_dim
+            dkv = torch.cat([dkv[: s.kv_rank], _deinterleave(dkv[s.kv_rank:], rd)], 0)
+            uq = uq.view(s.heads, s.dim + s.rot_dim, -1)
+            uq = torch.cat([uq[:, : s.dim], _deinterleave(uq[:, s.dim:], rd)], 1).reshape(-1, uq.shape[-1])
+        parts = [get(prefix + "dq"), dkv] + ([get(prefix + "g")] if s.gate != "none" else [])
+        self.w_in = torch.cat(parts, 0).to(dev, dt).contiguous()
         self.q_norm = get(prefix + "dq.norm").to(dev, torch.float32)
         self.kv_norm = get(prefix + "dkv.norm").to(dev, torch.float32)
-        self.w_uq = get(prefix + "uq").to(dev, dt).contiguous()
+        self.w_uq = uq.to(dev, dt).contiguous()
         self.w_uk = get(prefix + "uk").to(dev, dt).view(s.heads, s.dim, s.kv_rank).contiguous()
         self.w_uv_t = get(prefix + "uv").to(dev, dt).view(s.heads, s.vdim, s.kv_rank).transpose(1, 2).contiguous()
         self.w_o = get(prefix + "o").to(dev, dt).contiguous()
@@ -104,21 +150,25 @@ class LatentAttention:
         def w(*shape, scale=1.0):
             return torch.randn(*shape, generator=gen) * std * scale
 
-        t = {"dq": w(s.q_rank, H), "dkv": w(s.key_dim, H), "g": w(s.heads, H),
+        t = {"dq": w(s.q_rank, H), "dkv": w(s.key_dim, H), "g": w(max(s.gate_size, 1), H, scale=4.0 if s.gate == "channel" else 1.0),
              "dq.norm": 1.0 + 0.1 * torch.randn(s.q_rank, generator=gen),
              "dkv.norm": 1.0 + 0.1 * torch.randn(s.kv_rank, generator=gen),
              "uq": w(s.heads * (s.dim + s.rot_dim), s.q_rank, scale=4.0), "uk": w(s.heads * s.dim, s.kv_rank, scale=4.0),
              "uv": w(s.heads * s.vdim, s.kv_rank, scale=4.0), "o": w(H, s.heads * s.vdim)}
+        if s.gate == "none":
+            del t["g"]
         self.load(lambda k: t[k], "")
         return t
 
     def cache_shape(self, num_blocks: int, block_size: int):
         return (num_blocks, block_size, self.spec.key_dim)
 
-    def forward(self, h: torch.Tensor, meta, cache: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, meta, cache: torch.Tensor, state=None) -> torch.Tensor:
         s, ops = self.spec, self.ops
         T = h.shape[0]
         proj = F.linear(h, self.w_in)
+        _side(self, proj)
+        gate_off = s.q_rank + s.key_dim
         cq = torch.empty(T, s.q_rank, device=h.device, dtype=h.dtype)
         ops.latent_prepare(cq, cache, proj, meta.positions, meta.slot_mapping, self.q_norm, self.kv_norm,
                            self.inv_freq, s.q_rank, s.kv_rank, s.rot_dim, self.eps)
@@ -134,8 +184,13 @@ class LatentAttention:
             q_abs = _mm32(qh[:, :, : s.dim].transpose(0, 1), self.w_uk)            # [heads, T, kv_rank] fp32
         o_lat = torch.empty(s.heads, T, s.kv_rank, device=h.device, dtype=h.dtype)
         ops.latent_attention(o_lat, q_abs, q, proj, cache, meta, self.inv_freq, s.heads, s.dim, s.rot_dim,
-                             s.kv_rank, s.q_rank + s.key_dim, s.scale, s.window)
+                             s.kv_rank, gate_off if s.gate == "head" else -1, s.scale, s.window)
         o = torch.bmm(o_lat, self.w_uv_t)                              # [heads, T, vdim]
+        if s.gate == "channel":
+            # heads side by side per token, each element times the sigmoid of its gate column: one pass
+            cat = torch.empty(T, s.heads * s.vdim, device=h.device, dtype=h.dtype)
+            ops.gate_mul(cat, o, proj[:, gate_off:gate_off + s.heads * s.vdim])
+            return F.linear(cat, self.w_o)
         return F.linear(o.transpose(0, 1).reshape(T, s.heads * s.vdim), self.w_o)
 
 
@@ -269,6 +324,7 @@ def _rand(gen, *shape, std=1.0):
 class WindowAttention:
     cache_dim = property(lambda self: self.spec.cache_dim)
     state_shapes = None
+    side_weight, side_rows, side_out = "w_in", 0, None
 
     def __init__(self, spec: WindowAttentionSpec, hidden: int, eps: float, device, dtype, ops):
         self.spec, self.hidden, self.eps, self.device, self.dtype, self.ops = spec, hidden, eps, device, dtype, ops
@@ -278,6 +334,7 @@ class WindowAttention:
         self.w_o = None      # [hidden, heads * vdim]
         self.b_o = None
         self.lam = 0.0       # differential attention: weight of the second map
+        self.sink_w = None   # fp32 [heads]: learned sink logits (``sink_weights``)
         half = spec.rot_dims // 2
         i = torch.arange(half, dtype=torch.float32)
         # f_i = base^(-2i / dims), 32-bit
@@ -308,6 +365,8 @@ class WindowAttention:
             # lam = exp(lq1 . lk1) - exp(lq2 . lk2) + diff, one number for the layer (32-bit)
             lq1, lk1, lq2, lk2 = (get(prefix + n).to(torch.float32) for n in ("lq1", "lk1", "lq2", "lk2"))
             self.lam = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum()) + torch.tensor(s.diff))
+        if s.sink_weights:
+            self.sink_w = get(prefix + "sink").to(dev, torch.float32).contiguous()
         self.w_o = get(prefix + "o").to(dev, dt).contiguous()
         if s.out_bias:
             self.b_o = get(prefix + "o.b").to(dev, dt).contiguous()
@@ -331,6 +390,8 @@ class WindowAttention:
             del t["k.norm"]
         if s.maps == 2:
             t.update({n: _rand(gen, s.dim, std=0.2) for n in ("lq1", "lk1", "lq2", "lk2")})
+        if s.sink_weights:
+            t["sink"] = _rand(gen, s.heads)
         return t
 
     def mix(self, h, meta, cache, state, out, out_scale: float = 1.0):
@@ -338,8 +399,9 @@ class WindowAttention:
         (a column slice of a wider buffer is fine)."""
         s, ops = self.spec, self.ops
         proj = F.linear(h, self.w_in, self.b_in)
+        _side(self, proj)
         ops.attn_prepare(proj, cache, meta, self.inv_freq, s, self.q_norm, self.k_norm, self.eps)
-        ops.window_attention(out, proj, cache, meta, s, self.gate_off, out_scale, self.lam, self.eps)
+        ops.window_attention(out, proj, cache, meta, s, self.gate_off, out_scale, self.lam, self.eps, self.sink_w)
         return out
 
     def forward(self, h, meta, cache, state):
@@ -509,6 +571,54 @@ class DeltaRule:
         return F.linear(self.mix(h, meta, cache, state, out), self.w_o)
 
 
+class MLstm:
+    cache_dim = 0
+    side_weight, side_rows, side_out = "w_in", 0, None
+
+    def __init__(self, spec: MLstmSpec, hidden: int, eps: float, device, dtype, ops):
+        self.spec, self.hidden, self.eps, self.device, self.dtype, self.ops = spec, hidden, eps, device, dtype, ops
+        self.w_in = None     # [q | k | v | gate, hidden]
+        self.w_if = None     # [input gate (heads) | forget gate (heads), hidden]; its product is 32-bit
+        self.b_if = None     # fp32 [2 * heads]
+        self.norm = None     # fp32 [heads * vdim]
+        self.w_o = None
+
+    @property
+    def out_size(self) -> int:
+        return self.spec.out_size
+
+    def state_shapes(self, slots: int):
+        """Matrix state, normaliser and running maximum of the log gates per sequence slot and head."""
+        s = self.spec
+        return [(slots, s.heads, s.dim, s.vdim), (slots, s.heads, s.dim), (slots, s.heads)]
+
+    def load(self, get, prefix: str):
+        dt, dev = self.dtype, self.device
+        self.w_in = torch.cat([get(prefix + n) for n in ("q", "k", "v", "g")], 0).to(dev, dt).contiguous()
+        self.w_if = torch.cat([get(prefix + "i"), get(prefix + "f")], 0).to(dev, dt).contiguous()
+        self.b_if = torch.cat([get(prefix + "i.b").float(), get(prefix + "f.b").float()]).to(dev).contiguous()
+        self.norm = get(prefix + "norm").to(dev, torch.float32).contiguous()
+        self.w_o = get(prefix + "o").to(dev, dt).contiguous()
+
+    def init_random(self, gen, std: float):
+        s, H = self.spec, self.hidden
+        qk = s.heads * s.dim
+        return {"q": _rand(gen, qk, H, std=std * 4), "k": _rand(gen, qk, H, std=std * 4),
+                "v": _rand(gen, s.out_size, H, std=std * 4), "g": _rand(gen, s.out_size, H, std=std * 4),
+                "i": _rand(gen, s.heads, H, std=std * 8), "f": _rand(gen, s.heads, H, std=std * 8),
+                "i.b": _rand(gen, s.heads), "f.b": _rand(gen, s.heads) + 2.0,
+                "norm": 1.0 + 0.2 * _rand(gen, s.out_size), "o": _rand(gen, H, s.out_size, std=std)}
+
+    def forward(self, h, meta, cache, state):
+        s = self.spec
+        proj = F.linear(h, self.w_in)
+        _side(self, proj)
+        gates = _linear32(h, self.w_if)                                # [T, 2 * heads], 32-bit
+        out = torch.empty(h.shape[0], s.out_size, device=h.device, dtype=h.dtype)
+        self.ops.mlstm(out, state, proj, gates, self.b_if, self.norm, s, self.eps, meta)
+        return F.linear(out, self.w_o)
+
+
 class ParallelMixer:
     """left_scale * left(h) + right_scale * right(h): both halves write their scaled head outputs
     into one [T, left | right] buffer; one GEMM with the concatenated output weights sums them."""
@@ -549,10 +659,13 @@ class ParallelMixer:
 
 
 class DenseFF:
-    def __init__(self, spec: DenseFFSpec, hidden: int, device, dtype, ops):
-        self.spec, self.hidden, self.device, self.dtype, self.ops = spec, hidden, device, dtype, ops
+    side_weight, side_rows, side_out = "w_up", 0, None
+
+    def __init__(self, spec: DenseFFSpec, hidden: int, device, dtype, ops, eps: float = 0.0):
+        self.spec, self.hidden, self.device, self.dtype, self.ops, self.eps = spec, hidden, device, dtype, ops, eps
         self.w_up = self.w_down = None
         self.c0 = self.c1 = 0.0     # xielu: softplus(p), 1/2 + softplus(q)
+        self.coef = None            # polynorm: fp32 [4] = a, b, c, e
 
     def load(self, get, prefix: str):
         dt, dev = self.dtype, self.device
@@ -561,15 +674,29 @@ class DenseFF:
         if self.spec.act == "xielu":
             sp = F.softplus(get(prefix + "act").to(torch.float32))
             self.c0, self.c1 = float(sp[0]), float(torch.tensor(0.5) + sp[1])
+        if self.spec.act == "polynorm":
+            self.coef = get(prefix + "act").to(dev, torch.float32).contiguous()
 
     def init_random(self, gen, std: float):
         t = {"up": _rand(gen, self.spec.ff, self.hidden, std=std * 4), "down": _rand(gen, self.hidden, self.spec.ff, std=std)}
         if self.spec.act == "xielu":
             t["act"] = _rand(gen, 2, std=0.5)
+        if self.spec.act == "polynorm":
+            t["act"] = _rand(gen, 4, std=0.5)
         return t
 
     def forward(self, h):
         up = F.linear(h, self.w_up)
+        _side(self, up)
+        ff = self.spec.ff
+        if self.spec.act == "polynorm":
+            act = torch.empty(h.shape[0], ff, device=h.device, dtype=h.dtype)
+            self.ops.polynorm(act, up[:, :ff], self.coef, self.eps)
+            return F.linear(act, self.w_down)
+        if self.side_rows:
+            act = torch.empty(h.shape[0], ff, device=h.device, dtype=h.dtype)
+            self.ops.activation(act, up[:, :ff], self.spec.act, self.c0, self.c1)
+            return F.linear(act, self.w_down)
         self.ops.activation(up, up, self.spec.act, self.c0, self.c1)
         return F.linear(up, self.w_down)
 
@@ -579,6 +706,8 @@ class RoutedMoE:
     which the residual update (``add_normed``) combines: row ``pair_slot[t * top + j]`` of ``ye`` is the
     output of token t's j-th choice ``ids[t, j]`` (a value >= experts is an identity expert: the token's
     own input), weighted ``wts[t, j]``; ``shared`` is the shared expert's output or None."""
+
+    side_weight, side_rows, side_out = "ws_gu", 0, None
 
     def __init__(self, spec: RoutedMoESpec, hidden: int, device, dtype, ops):
         self.spec, self.hidden, self.device, self.dtype, self.ops = spec, hidden, device, dtype, ops
@@ -617,7 +746,8 @@ class RoutedMoE:
         T, dev = h.shape[0], h.device
         ids = torch.empty(T, s.top, dtype=torch.int32, device=dev)
         wts = torch.empty(T, s.top, dtype=torch.float32, device=dev)
-        ops.route_topk(ids, wts, _linear32(h, self.w_router), self.correction, s.top, s.scale, s.experts)
+        ops.route_topk(ids, wts, _linear32(h, self.w_router), self.correction, s.top, s.scale, s.experts,
+                       s.groups, s.keep_groups, s.renorm)
         # the identity experts share one bucket (s.experts) that no GEMM tile serves
         P, nb = T * s.top, s.experts + (1 if s.identity else 0)
         if self._packed_ok(h, P, nb):
@@ -636,11 +766,16 @@ class RoutedMoE:
         return ye, pair_slot, ids, wts, s.experts, h, self._shared(h)
 
     def _shared(self, h: torch.Tensor):
-        if not self.spec.shared_ff:
+        """The shared expert's output (None without one); the side projection rides on its gate | up GEMM."""
+        n = self.spec.shared_ff
+        if not n and not self.side_rows:
             return None
         g = F.linear(h, self.ws_gu)
-        a = torch.empty(h.shape[0], self.spec.shared_ff, device=h.device, dtype=h.dtype)
-        self.ops.activation(a, g, "silu_mul")
+        _side(self, g)
+        if not n:
+            return None
+        a = torch.empty(h.shape[0], n, device=h.device, dtype=h.dtype)
+        self.ops.activation(a, g[:, :2 * n], "silu_mul")
         return F.linear(a, self.ws_down)
 
     def _packed_ok(self, h: torch.Tensor, P: int, nb: int) -> bool:
@@ -683,10 +818,10 @@ class RoutedMoE:
         return ye, pair_slot
 
 
-def make_ff(spec, hidden: int, device, dtype, ops):
+def make_ff(spec, hidden: int, device, dtype, ops, eps: float = 0.0):
     """The weight holder of a feed-forward spec that takes no token ids."""
     if isinstance(spec, DenseFFSpec):
-        return DenseFF(spec, hidden, device, dtype, ops)
+        return DenseFF(spec, hidden, device, dtype, ops, eps)
     if isinstance(spec, RoutedMoESpec):
         return RoutedMoE(spec, hidden, device, dtype, ops)
     raise NotImplementedError(type(spec).__name__)
@@ -702,6 +837,8 @@ def make_mixer(spec, hidden: int, eps: float, device, dtype, ops):
         return GatedDelta(spec, hidden, eps, device, dtype, ops)
     if isinstance(spec, DeltaRuleSpec):
         return DeltaRule(spec, hidden, eps, device, dtype, ops)
+    if isinstance(spec, MLstmSpec):
+        return MLstm(spec, hidden, eps, device, dtype, ops)
     if isinstance(spec, ParallelMixerSpec):
         return ParallelMixer(spec, hidden, eps, device, dtype, ops)
     if isinstance(spec, LatentAttentionSpec):

@@ -23,6 +23,7 @@ ARCHITECTURES = {
     "kesirax": ("hipserve.models.kesirax", "KesiraxModel", "hipserve.weights.safetensors_loader:load_named_tensors"),
     "fikizen": ("hipserve.models.fikizen", "FikizenModel", "hipserve.weights.safetensors_loader:load_named_tensors"),
     "kemavik": ("hipserve.models.kemavik", "KemavikModel", "hipserve.weights.safetensors_loader:load_named_tensors"),
+    "topezen": ("hipserve.models.topezen", "TopezenModel", "hipserve.weights.safetensors_loader:load_named_tensors"),
 }
 
 

@@ -515,8 +515,24 @@ class ReferenceOps:
     def attn_prepare(self, proj, cache, meta, inv_freq, sp, q_norm, k_norm, eps):
         ref.attn_prepare(proj, cache, meta.positions, meta.slot_mapping, inv_freq, sp, q_norm, k_norm, eps)
 
-    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0, lam=0.0, eps=0.0):
-        ref.window_attention(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, sp, gate_off, out_scale, lam, eps)
+    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0, lam=0.0, eps=0.0, sink_w=None):
+        ref.window_attention(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, sp, gate_off, out_scale, lam, eps,
+                             sink_w)
+
+    def gated_add_norms(self, out1, out2, residual, w1, w2, eps, first=None, second=None):
+        ref.gated_add_norms(out1, out2, residual, w1, w2, eps, first, second)
+
+    def polynorm(self, out, x, coef, eps):
+        ref.polynorm(out, x, coef, eps)
+        return out
+
+    def gate_mul(self, out, x, gate):
+        ref.gate_mul(out, x, gate)
+        return out
+
+    def mlstm(self, out, state, proj, gates, b_if, norm_w, sp, eps, meta):
+        ref.mlstm(out, state[0], state[1], state[2], proj, gates, b_if, norm_w, sp, eps, meta.seq_cu, meta.seq_ctx,
+                  meta.seq_state)
 
     def add_normed(self, out, residual, y, w, eps, moe=None):
         ref.add_normed(out, residual, y, w, eps, moe)
@@ -533,8 +549,8 @@ class ReferenceOps:
         wl = torch.nn.functional.linear(t.float(), w2.float())
         ref.wkv(out, state, proj, wl, w0, u, norm_w, sp, eps, meta.seq_cu, meta.seq_ctx, meta.seq_state)
 
-    def route_topk(self, ids, wts, logits, correction, top, scale, E):
-        ref.route_topk(ids, wts, logits, correction, top, scale, E)
+    def route_topk(self, ids, wts, logits, correction, top, scale, E, groups=1, keep_groups=1, renorm=False):
+        ref.route_topk(ids, wts, logits, correction, top, scale, E, groups, keep_groups, renorm)
 
     def gated_delta(self, y, state, proj, conv_w, a_log, dt_bias, norm_w, sp, eps, meta):
         ref.gated_delta(y, state[0], state[1], proj, conv_w, a_log, dt_bias, norm_w, sp, eps, meta.seq_cu,

@@ -447,7 +447,7 @@ def latent_attention(o_lat, q_abs, q, proj, cache, seq_cu, seq_ctx, seq_bt, inv_
     """Per sequence s with rows cu[s]..cu[s+1]-1 at positions ctx[s] - n .. ctx[s] - 1: scores of
     head h = (q_abs[h, t] . latent + RoPE(q[t, h, dim:]) . rotary key) * scale over the keys
     0 <= pos - j < window (window 0: all j <= pos), softmax, latent-space output times
-    sigmoid(proj[t, gate_off + h])."""
+    sigmoid(proj[t, gate_off + h]) (gate_off >= 0)."""
     bs = cache.shape[1]
     flat = cache.view(-1, cache.shape[-1])
     cu = [int(v) for v in seq_cu]
@@ -470,8 +470,9 @@ def latent_attention(o_lat, q_abs, q, proj, cache, seq_cu, seq_ctx, seq_bt, inv_
         ok = (d >= 0) & ((d < window) if window > 0 else (d >= 0))
         sc = sc.masked_fill(~ok, float("-inf"))
         o = torch.einsum("hnj,jk->hnk", torch.softmax(sc, -1), kv[:, :kv_rank])
-        g = torch.sigmoid(proj[a:b, gate_off:gate_off + heads].float())   # [n, heads]
-        o_lat[:, a:b] = (o * g.t().unsqueeze(-1)).to(o_lat.dtype)
+        if gate_off >= 0:
+            o = o * torch.sigmoid(proj[a:b, gate_off:gate_off + heads].float()).t().unsqueeze(-1)   # [heads, n, 1]
+        o_lat[:, a:b] = o.to(o_lat.dtype)
 
 
 def mingru_scan(y, state, proj, b_z, b_x, seq_cu, seq_ctx, seq_state):
@@ -578,10 +579,12 @@ def attn_prepare(proj, cache, positions, slots, inv_freq, sp, q_norm, k_norm, ep
     cache.view(-1, cache.shape[-1])[slots[ok]] = torch.cat([k, v], -1).to(cache.dtype)[ok]
 
 
-def window_attention(out, proj, cache, seq_cu, seq_ctx, seq_bt, sp, gate_off, out_scale, lam=0.0, eps=0.0):
+def window_attention(out, proj, cache, seq_cu, seq_ctx, seq_bt, sp, gate_off, out_scale, lam=0.0, eps=0.0, sink_w=None):
     """Per sequence s (rows cu[s]..cu[s+1]-1 at positions ctx[s]-n .. ctx[s]-1): head h scores
     its prepared query against the cached keys of head h // (heads / kv_heads) with
-    0 <= pos - j < window; weights exp(s_j) / (sink + sum exp(s_j)); out[t, h * vdim ..] =
+    0 <= pos - j < window or j < sp.keep_first; scores s_j = q . k * scale, then
+    softcap * tanh(s_j / softcap) (softcap > 0); weights exp(s_j) / (sink + sum exp(s_j)) with
+    sink = exp(sink_w[h]) (1 without weights); out[t, h * vdim ..] =
     weighted values * sigmoid(proj[t, gate_off + h]) (gate_off >= 0) * out_scale.
     ``sp.maps`` = 2: query and key heads hold [map 1 | map 2]; the head output is
     o = a1 - lam * a2 of the two maps' weighted values, o / sqrt(mean(o^2) + eps) * (1 - sp.diff)."""
@@ -595,7 +598,7 @@ def window_attention(out, proj, cache, seq_cu, seq_ctx, seq_bt, sp, gate_off, ou
             continue
         ctx = int(seq_ctx[s])
         pos = torch.arange(ctx - (b - a), ctx, device=proj.device)
-        lo = 0 if W <= 0 else max(0, int(pos[0]) - W + 1)
+        lo = 0 if (W <= 0 or sp.keep_first > 0) else max(0, int(pos[0]) - W + 1)
         j = torch.arange(lo, ctx, device=proj.device)
         kv = flat[seq_bt[s].long()[j // bs] * bs + j % bs].float()
         k = kv[:, :G * M * d].view(-1, G, M * d).repeat_interleave(H // G, 1).reshape(-1, H * M, d)
@@ -603,14 +606,19 @@ def window_attention(out, proj, cache, seq_cu, seq_ctx, seq_bt, sp, gate_off, ou
         v = v.repeat_interleave(M, 1)
         q = proj[a:b, :H * M * d].float().view(b - a, H * M, d)
         sc = torch.einsum("nhd,jhd->hnj", q, k) * sp.scale
+        if sp.softcap > 0:
+            sc = torch.tanh(sc / sp.softcap) * sp.softcap
         dd = pos[:, None] - j[None]
-        ok = (dd >= 0) & ((dd < W) if W > 0 else (dd >= 0))
+        ok = (dd >= 0) & (((dd < W) | (j[None] < sp.keep_first)) if W > 0 else (dd >= 0))
         sc = sc.masked_fill(~ok, float("-inf"))
         m = sc.max(-1, keepdim=True).values
+        sk = 0.0   # the sink's logit: a key without a value
+        if sp.sink and sink_w is not None:
+            sk = sink_w.float().repeat_interleave(M).view(H * M, 1, 1)
         if sp.sink:
-            m = m.clamp(min=0.0)
+            m = torch.maximum(m, torch.as_tensor(sk, dtype=m.dtype, device=m.device))
         e = torch.exp(sc - m)
-        den = e.sum(-1, keepdim=True) + (torch.exp(-m) if sp.sink else 0.0)
+        den = e.sum(-1, keepdim=True) + (torch.exp(sk - m) if sp.sink else 0.0)
         o = torch.einsum("hnj,jhv->nhv", e / den, v)
         if M == 2:
             o = o.view(b - a, H, 2, dv)
@@ -784,12 +792,106 @@ def wkv(out, S, proj, wl, w0, u, norm_w, sp, eps, seq_cu, seq_ctx, seq_state):
         out[a0:b0] = (_rows_rms(o, eps).reshape(n, N) * norm_w.float() * (g * torch.sigmoid(g))).to(out.dtype)
 
 
-def route_topk(ids, wts, logits, correction, top, scale, E):
+def route_topk(ids, wts, logits, correction, top, scale, E, groups=1, keep_groups=1, renorm=False):
     """s = softmax(logits) (fp32, over all router outputs); the ``top`` outputs with the largest
     s + correction are chosen (ties: the lower index); wts = s * scale of the chosen, ids = their
-    index, outputs >= E (experts without weights) all written as E."""
+    index, outputs >= E (experts without weights) all written as E. ``groups`` > 1: the outputs
+    form equal groups of neighbours, a group scores its largest s + correction, and outputs
+    outside the ``keep_groups`` best groups cannot be chosen. ``renorm``: the chosen s are divided
+    by their sum (+ 1e-20) before the scaling."""
     s = torch.softmax(logits.float(), -1)
     c = s + correction.float()
+    if groups > 1:
+        T, n = c.shape
+        best = c.view(T, groups, n // groups).max(-1).values
+        kept = torch.argsort(-best, dim=-1, stable=True)[:, :keep_groups]
+        allow = torch.zeros_like(best, dtype=torch.bool).scatter_(1, kept, True)
+        c = c.masked_fill(~allow.repeat_interleave(n // groups, 1), float("-inf"))
     order = torch.argsort(-c, dim=-1, stable=True)[:, :top]
-    wts.copy_(s.gather(1, order) * scale)
+    w = s.gather(1, order)
+    if renorm:
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    wts.copy_(w * scale)
     ids.copy_(order.clamp(max=E).to(ids.dtype))
+
+
+# ---------------------------------------------------------------------------------
+# parallel blocks with gated sublayer results and two single-weight norms, PolyNorm, the
+# per-channel output gate of heads stored head-major, the mLSTM matrix memory over state slots
+
+def gated_add_norms(out1, out2, residual, w1, w2, eps, first=None, second=None):
+    """residual (fp32, in place) += sum over the given sublayers of sigmoid(g + b) * y, each
+    ``(y, g, b)`` with y [T, H] the sublayer's result (or the parts of a mixture's output,
+    ``(ye, pair_slot, wts, shared)``: y[t] = shared[t] + sum_j wts[t, j] * ye[pair_slot[t * top + j]]),
+    g [T, H] its gate's pre-activation (any row stride) and b [H] the gate's bias. Then
+    out1 = residual / rms * w1 and out2 = residual / rms * w2 (w: one number or H; out2 / w2 may be None)."""
+    for sub in (first, second):
+        if sub is None:
+            continue
+        y, g, b = sub
+        if isinstance(y, tuple):
+            ye, pair_slot, wts, shared = y
+            T, top = wts.shape
+            rows = ye.float().index_select(0, pair_slot.long().clamp(min=0)).view(T, top, -1)
+            y = (rows * wts.float().unsqueeze(-1)).sum(1)
+            if shared is not None:
+                y = y + shared.float()
+        residual += torch.sigmoid(g.float() + b.float()) * y.float()
+    n = _rows_rms(residual, eps)
+    out1.copy_((n * w1.float()).to(out1.dtype))
+    if out2 is not None:
+        out2.copy_((n * w2.float()).to(out2.dtype))
+
+
+def polynorm(out, x, coef, eps):
+    """out = a N(z) + b N(z^2) + c N(z^3) + e over every row z of x, N(u) = u / sqrt(mean(u^2) + eps),
+    coef = [a, b, c, e] (fp32)."""
+    z = x.float()
+    a, b, c, e = (coef[i].float() for i in range(4))
+    out.copy_((a * _rows_rms(z, eps) + b * _rows_rms(z * z, eps) + c * _rows_rms(z * z * z, eps) + e).to(out.dtype))
+
+
+def gate_mul(out, x, gate):
+    """out[t, h * d + j] = x[h, t, j] * sigmoid(gate[t, h * d + j]) for x [heads, T, d] (head-major)."""
+    Hh, T, d = x.shape
+    out.copy_((x.float().transpose(0, 1).reshape(T, Hh * d) * torch.sigmoid(gate.float())).to(out.dtype))
+
+
+def mlstm(out, S, N, M, proj, gates, b_if, norm_w, sp, eps, seq_cu, seq_ctx, seq_state):
+    """proj rows = [q | k | v | gate | ...], gates (fp32) rows = [input gate | forget gate] pre-activations per head.
+    Per head, from the sequence's slot (zeros when the step starts at position 0), with
+    i = cap tanh((. + b) / cap), f = logsigmoid(cap tanh((. + b) / cap)), q scaled by dim^-1/2:
+      m' = max(f + m, i);  S = e^(f + m - m') S + e^(i - m') k v^T;  n likewise with k;  m = m'
+      o = S^T q / (max(|n . q|, e^-m) + 1e-6)
+    out = o / rms(o) per head * norm_w * sigmoid(gate). S [slots, heads, dim, vdim], N [slots, heads, dim], M [slots, heads]."""
+    H, d, dv, cap = sp.heads, sp.dim, sp.vdim, sp.gate_cap
+    cu = [int(x) for x in seq_cu]
+    for s in range(len(cu) - 1):
+        a0, b0 = cu[s], cu[s + 1]
+        n = b0 - a0
+        if n == 0:
+            continue
+        slot, start = int(seq_state[s]), int(seq_ctx[s]) - n
+        p = proj[a0:b0].float()
+        q = p[:, :H * d].view(n, H, d) * d ** -0.5
+        k = p[:, H * d:2 * H * d].view(n, H, d)
+        v = p[:, 2 * H * d:2 * H * d + H * dv].view(n, H, dv)
+        gate = p[:, 2 * H * d + H * dv:2 * H * d + 2 * H * dv]
+        pre = gates[a0:b0].float() + b_if.float()
+        ig = cap * torch.tanh(pre[:, :H] / cap)
+        fg = torch.nn.functional.logsigmoid(cap * torch.tanh(pre[:, H:] / cap))
+        if start > 0:
+            st, nn, mm = S[slot].clone(), N[slot].clone(), M[slot].clone()
+        else:
+            st, nn, mm = torch.zeros_like(S[slot]), torch.zeros_like(N[slot]), torch.zeros_like(M[slot])
+        o = torch.empty(n, H, dv, device=proj.device)
+        for t in range(n):
+            m_new = torch.maximum(fg[t] + mm, ig[t])
+            fa, fb = torch.exp(fg[t] + mm - m_new), torch.exp(ig[t] - m_new)
+            st = fa[:, None, None] * st + fb[:, None, None] * k[t, :, :, None] * v[t, :, None, :]
+            nn = fa[:, None] * nn + fb[:, None] * k[t]
+            mm = m_new
+            den = torch.maximum((nn * q[t]).sum(-1).abs(), torch.exp(-mm)) + 1e-6
+            o[t] = torch.einsum("hkv,hk->hv", st, q[t]) / den[:, None]
+        S[slot], N[slot], M[slot] = st, nn, mm
+        out[a0:b0] = (_rows_rms(o, eps).reshape(n, H * dv) * norm_w.float() * torch.sigmoid(gate)).to(out.dtype)
