@@ -63,10 +63,12 @@ void launch_add_normed(void* out, float* residual, const float* w, int T, int H,
                        const void* h, const void* shared, bool f32, hipStream_t s);
 
 // Softmax router (router.hip): s = softmax(logits[T, n]); the `top` largest s + correction are chosen (ties: the
-// lower index); ids[T, top] = min(index, E), wts[T, top] = s * scale.
+// lower index); ids[T, top] = min(index, E), wts[T, top] = s * scale. groups > 1: only outputs of the `keep`
+// groups (of n / groups neighbours) with the largest s + correction can be chosen; renorm: the chosen s are
+// divided by their sum + 1e-20 first.
 int route_topk_max_outputs();
 void launch_route_topk(int* ids, float* wts, const float* logits, const float* correction, int T, int n, int top,
-                       float scale, int E, hipStream_t s);
+                       float scale, int E, int groups, int keep, bool renorm, hipStream_t s);
 
 // Window attention on a paged cache [blocks, block_size, kv_heads * dim | kv_heads * vdim] (window_attention.hip).
 // attn_prepare: per row of proj = [q | k | v | ...]: optional RMS norm of q and k (norm_mode 0: none; 1: over the
@@ -78,8 +80,10 @@ void launch_attn_prepare(void* proj, long ld, void* cache, const long* positions
                          const float* inv_freq, int nfreq, int T, int heads, int kv_heads, int maps, int dim, int vdim,
                          const float* q_norm, const float* k_norm, int norm_mode, bool v_norm, float eps, bool f32,
                          hipStream_t s);
-// Sequences seq0 .. seq1-1 of the step, `tq` tokens per workgroup: keys 0 <= pos - j < window (0: all),
-// weights exp(s_j) / (sink + sum exp), head output times sigmoid(proj[t, gate_off + h]) (gate_off >= 0) and
+// Sequences seq0 .. seq1-1 of the step, `tq` tokens per workgroup: keys 0 <= pos - j < window (0: all) or
+// j < keep, scores q . k * scale, through softcap * tanh(. / softcap) when softcap > 0,
+// weights exp(s_j) / (sink + sum exp) with sink = exp(sink_w[h]) (1 when sink_w is null),
+// head output times sigmoid(proj[t, gate_off + h]) (gate_off >= 0) and
 // out_scale into out[t * out_ld + h * vdim ..]. maps = 2 (differential attention): queries and keys hold
 // [map 1 | map 2] per head; the head output is o = a1 - lam a2, o / sqrt(mean(o^2) + eps) * post.
 int window_attention_max_vdim();
@@ -87,7 +91,7 @@ void launch_window_attention(void* out, long out_ld, const void* proj, long proj
                              const int* seq_cu, const int* seq_ctx, const int* seq_bt, int bt_width, int seq0, int seq1,
                              int rows_bound, int tq, int heads, int kv_heads, int dim, int vdim, int gate_off,
                              float scale, int window, bool sink, float out_scale, int maps, float lam, float post,
-                             float eps, bool f32, hipStream_t s);
+                             float eps, int keep, float softcap, const float* sink_w, bool f32, hipStream_t s);
 
 // bf16 on the matrix cores (window_attention_mfma.hip): 64 (token, head) rows of one key/value head per
 // workgroup, 32-key tiles. nparts > 1 (rows of one token each, rows_bound of them from batch row row_base on):
@@ -100,7 +104,8 @@ void launch_window_attention_mfma(void* out, long out_ld, const void* proj, long
                                   int bt_width, int seq0, int seq1, int rows_bound, int heads, int kv_heads, int dim,
                                   int vdim, int gate_off, float scale, int window, bool sink, float out_scale,
                                   int nparts, int part_keys, float* ws_acc, float* ws_ml, int row_base, int maps,
-                                  float lam, float post, float eps, hipStream_t s);
+                                  float lam, float post, float eps, int keep, float softcap, const float* sink_w,
+                                  hipStream_t s);
 
 // Delta-rule recurrences over state slots (delta_scan.hip). scratch: fp32, T * (2 * kv_heads * dim +
 // 2 * heads * vdim + 2 * heads) floats for the gated rule, T * 7 * heads * dim for the generalized one.
@@ -133,5 +138,30 @@ void launch_wkv_step(void* out, float* S, const void* proj, long T, const void* 
 // 3: x rows = [gate | up] of `cols` each, out = silu(gate) * up.
 void launch_activation(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, int kind, float c0,
                        float c1, bool f32, hipStream_t s);
+
+// Per row z of x: out = a N(z) + b N(z^2) + c N(z^3) + e, N(u) = u / sqrt(mean(u^2) + eps), coef = [a, b, c, e].
+void launch_polynorm(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, const float* coef,
+                     float eps, bool f32, hipStream_t s);
+// out[t, h * d + j] = x[h, t, j] * sigmoid(gate[t * gate_ld + h * d + j]) for x [heads, rows, d].
+void launch_gate_mul(void* out, const void* x, const void* gate, long gate_ld, int rows, int heads, int d, bool f32,
+                     hipStream_t s);
+
+// Parallel block with gated sublayer results and the next norms (gated_block.hip): residual[T, H] (fp32, in place)
+// += sigmoid(g1 + b1) * y1 + sigmoid(g2 + b2) * y2, y2 a row or (y2 null) shared + sum_j wts[t, j] ye[pair_slot[t top + j]];
+// out1 = residual / rms * w1, out2 (may be null) = residual / rms * w2; w1n / w2n: 1 or H weights.
+void launch_gated_add_norms(void* out1, void* out2, float* residual, const float* w1, int w1n, const float* w2, int w2n,
+                            int T, int H, float eps, const void* y1, const void* g1, long g1_ld, const float* b1,
+                            const void* y2, const void* g2, long g2_ld, const float* b2, const void* ye,
+                            const int* pair_slot, const float* wts, int top, const void* shared, bool f32,
+                            hipStream_t s);
+
+// mLSTM matrix memory over state slots (mlstm.hip): proj rows = [q | k | v | gate | ...], gates fp32 [T, 2 heads] =
+// [input | forget] pre-activations, b_if their biases, S [slots, heads, dim, vdim], N [slots, heads, dim],
+// M [slots, heads]; scratch: T * heads * (vdim + 5) floats. one_row_seqs: every sequence brings one row.
+int mlstm_max_dim();
+void launch_mlstm(void* out, float* S, float* N, float* M, const void* proj, long ld, const float* gates,
+                  const float* b_if, const float* norm_w, const int* seq_cu, const int* seq_ctx, const int* seq_state,
+                  int nseq, int T, float* scratch, int heads, int dim, int vdim, float cap, float eps,
+                  bool one_row_seqs, bool f32, hipStream_t s);
 
 }  // namespace hipserve

@@ -11,6 +11,21 @@
 
 namespace hipserve_shared {
 
+inline hipStream_t cur_stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
+
+#define CHECK_DEV(x) TORCH_CHECK((x).is_cuda(), #x " must be a GPU tensor")
+#define CHECK_CONTIG(x) TORCH_CHECK((x).is_contiguous(), #x " must be contiguous")
+#define CHECK_F32(x) TORCH_CHECK((x).scalar_type() == at::kFloat && (x).is_contiguous(), #x " must be contiguous fp32")
+#define CHECK_I32(x) TORCH_CHECK((x).scalar_type() == at::kInt && (x).is_contiguous(), #x " must be contiguous int32")
+
+inline bool is_f32(const at::Tensor& t, const char* who) {
+  TORCH_CHECK(t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16, who, ": bf16 or fp32 activations");
+  return t.scalar_type() == at::kFloat;
+}
+
+inline const void* opt_ptr(const c10::optional<at::Tensor>& t) { return t.has_value() ? t->data_ptr() : nullptr; }
+inline bool rows2d(const at::Tensor& t) { return t.dim() == 2 && t.stride(1) == 1; }
+
 inline void moe_align(const at::Tensor& ids, int64_t E, int64_t tile, at::Tensor& slots, at::Tensor& tile_expert,
                       at::Tensor& pair_slot) {
   auto i32 = [](const at::Tensor& t) { return t.scalar_type() == at::kInt && t.is_contiguous(); };

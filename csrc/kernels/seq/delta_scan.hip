@@ -586,45 +586,6 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ out, long out_ld, const T* __restrict__ x,
-                                                         long x_ld, int cols, int kind, float c0, float c1) {
-  const long t = blockIdx.x;
-  const int c = blockIdx.y * 256 + threadIdx.x;
-  if (c >= cols) return;
-  const float z = ldf<T>(x, t * x_ld + c);
-  float r;
-  if (kind == 0) r = tanhf(z);
-  else if (kind == 2) { r = fmaxf(z, 0.f); r *= r; }
-  else if (kind == 3) r = z * sigmoid_f(z) * ldf<T>(x, t * x_ld + cols + c);   // x rows = [gate | up]
-  else r = z > 0.f ? c0 * z * z + 0.5f * z : c1 * (expm1f(z) - z) + 0.5f * z;
-  stf<T>(out, t * out_ld + c, r);
-}
-
-// bf16 rows whose length, strides and base addresses are multiples of 8 elements: 8 elements per thread.
-__global__ __launch_bounds__(256) void activation_vec_kernel(unsigned short* __restrict__ out, long out_ld,
-                                                             const unsigned short* __restrict__ x, long x_ld,
-                                                             int cols8, int kind, float c0, float c1) {
-  const long t = blockIdx.x;
-  const int c = blockIdx.y * 256 + threadIdx.x;
-  if (c >= cols8) return;
-  const u16x8 z8 = *reinterpret_cast<const u16x8*>(x + t * x_ld + 8 * c);
-  u16x8 u8 = z8;
-  if (kind == 3) u8 = *reinterpret_cast<const u16x8*>(x + t * x_ld + 8 * (cols8 + c));
-  u16x8 r8;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float z = bf16_to_f32(z8[e]);
-    float r;
-    if (kind == 0) r = tanhf(z);
-    else if (kind == 2) { r = fmaxf(z, 0.f); r *= r; }
-    else if (kind == 3) r = z * sigmoid_f(z) * bf16_to_f32(u8[e]);
-    else r = z > 0.f ? c0 * z * z + 0.5f * z : c1 * (expm1f(z) - z) + 0.5f * z;
-    r8[e] = f32_to_bf16(r);
-  }
-  *reinterpret_cast<u16x8*>(out + t * out_ld + 8 * c) = r8;
-}
-
-template <typename T>
 void head_norm_gate(void* out, long out_ld, const float* o, const void* proj, long ld, int gate_off, const float* w,
                     int w_stride, int rows, int heads, int vdim, float eps, bool silu, float scale, hipStream_t s) {
   const long n = (long)rows * heads;
@@ -774,19 +735,6 @@ void launch_wkv_step(void* out, float* S, const void* proj, long T, const void* 
     wkv_step_kernel<unsigned short><<<grid, 256, smem, s>>>(
         (unsigned short*)out, S, (const unsigned short*)proj, T, (const unsigned short*)low, (const unsigned short*)w2,
         rank, w0, u, norm_w, seq_cu, seq_ctx, seq_state, heads, dim, eps);
-}
-
-void launch_activation(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, int kind, float c0,
-                       float c1, bool f32, hipStream_t s) {
-  if (rows <= 0 || cols <= 0) return;
-  dim3 grid(rows, (cols + 255) / 256);
-  if (f32) activation_kernel<float><<<grid, 256, 0, s>>>((float*)out, out_ld, (const float*)x, x_ld, cols, kind, c0, c1);
-  else if (cols % 8 == 0 && out_ld % 8 == 0 && x_ld % 8 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)x % 16 == 0)
-    activation_vec_kernel<<<dim3(rows, (cols / 8 + 255) / 256), 256, 0, s>>>(
-        (unsigned short*)out, out_ld, (const unsigned short*)x, x_ld, cols / 8, kind, c0, c1);
-  else
-    activation_kernel<unsigned short><<<grid, 256, 0, s>>>((unsigned short*)out, out_ld, (const unsigned short*)x, x_ld,
-                                                           cols, kind, c0, c1);
 }
 
 }  // namespace hipserve

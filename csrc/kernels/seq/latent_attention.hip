@@ -188,7 +188,7 @@ __global__ __launch_bounds__(64 * kMaxRows) void latent_attention_kernel(
     }
   }
   if (!active) return;
-  const float g = sigmoid_f(ldf<T>(proj, (long)trow * proj_ld + gate_off + head));
+  const float g = gate_off >= 0 ? sigmoid_f(ldf<T>(proj, (long)trow * proj_ld + gate_off + head)) : 1.f;
   const float inv = l > 0.f ? g / l : 0.f;
   T* dst = o_lat + ((long)head * T_rows + trow) * kv_rank;
 #pragma unroll

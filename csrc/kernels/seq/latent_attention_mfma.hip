@@ -247,8 +247,8 @@ __global__ __launch_bounds__(64 * NW, 2) void latent_attention_mfma_kernel(
       ws_ml[2 * wrow] = m_lds[tid];
       ws_ml[2 * wrow + 1] = l_lds[tid];
     } else if (act && l_lds[tid] > 0.f) {
-      const float gt = bf16_to_f32(proj[(long)(r0 + tok0 + rt) * proj_ld + gate_off + h0 + rh]);
-      f = sigmoid_f(gt) / l_lds[tid];
+      f = 1.f / l_lds[tid];
+      if (gate_off >= 0) f *= sigmoid_f(bf16_to_f32(proj[(long)(r0 + tok0 + rt) * proj_ld + gate_off + h0 + rh]));
     }
     alpha[tid] = f;
   }
@@ -293,7 +293,7 @@ __global__ __launch_bounds__(128) void latent_attention_reduce_kernel(
     const float M = wave_max(m);
     const float e = m > -INFINITY ? __expf(m - M) : 0.f;
     const float L = wave_sum(l * e);
-    const float gate = sigmoid_f(bf16_to_f32(proj[(long)(row_base + r) * proj_ld + gate_off + h]));
+    const float gate = gate_off >= 0 ? sigmoid_f(bf16_to_f32(proj[(long)(row_base + r) * proj_ld + gate_off + h])) : 1.f;
     sc[tid] = L > 0.f ? e * gate / L : 0.f;
   }
   __syncthreads();

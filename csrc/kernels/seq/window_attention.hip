@@ -18,8 +18,13 @@
 // window_attention: one wave per (token, query head) row; a workgroup holds `tq` tokens x the
 // query heads of ONE key/value head, so each 64-key tile is staged once for all of them. Scores:
 // lane = key, the head's key dims staged in chunks of 64 through LDS; online softmax per wave;
-// output: lane = value dim. With the sink the running (max, sum) start at (0, 1): a key of score
-// 0 without a value. Scores, softmax and accumulation are fp32 for both element types.
+// output: lane = value dim. With the sink the running (max, sum) start at (sink logit, 1): a key
+// without a value whose score is a learned number per head (0 without sink weights). Options:
+// softcap > 0 passes the scaled scores through softcap * tanh(. / softcap); keep > 0 keeps the
+// sequence's first `keep` keys visible behind the window. The kernel then walks a compacted key
+// index u: the kept keys below the workgroup's window first (u < nk), then the window's keys
+// (key = u - nk + lo), so tiles, runs of keys and the split over workgroups need no second loop.
+// Scores, softmax and accumulation are fp32 for both element types.
 #include "seq_common.h"
 #include "hipserve/seq_kernels.h"
 
@@ -142,7 +147,8 @@ __global__ __launch_bounds__(64 * kMaxRows) void window_attention_kernel(
     T* __restrict__ out, long out_ld, const T* __restrict__ proj, long proj_ld, const T* __restrict__ cache,
     int block_size, const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx, const int* __restrict__ seq_bt,
     int bt_width, int seq0, int seq1, int tq, int hc, int hchunks, int heads, int kv_heads, int dim, int vdim,
-    int gate_off, float scale, int window, bool sink, float out_scale, float lam, float post, float eps) {
+    int gate_off, float scale, int window, bool sink, float out_scale, float lam, float post, float eps, int keep,
+    float softcap, const float* __restrict__ sink_w) {
   extern __shared__ float sm[];
   const int nrows = blockDim.x >> 6;
   const int qd = MAPS * dim;                       // a row's query elements
@@ -172,24 +178,30 @@ __global__ __launch_bounds__(64 * kMaxRows) void window_attention_kernel(
   const int p_first = ctx - n + tok0, p_last = p_first + ntok - 1;
   const int lo = window > 0 ? max(0, p_first - window + 1) : 0;
   const int my_lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int nk = (window > 0 && keep > 0) ? min(keep, lo) : 0;   // kept keys below the workgroup's window
+  const int total = nk + p_last - lo + 1;
+  const float sink0 = (sink && sink_w != nullptr) ? sink_w[head] : 0.f;
+  const float icap = softcap > 0.f ? 1.f / softcap : 0.f;
   float m[MAPS], l[MAPS], acc[MAPS][kMaxCh];
 #pragma unroll
   for (int mp = 0; mp < MAPS; ++mp) {
-    m[mp] = sink ? 0.f : -INFINITY;
+    m[mp] = sink ? sink0 : -INFINITY;
     l[mp] = sink ? 1.f : 0.f;
 #pragma unroll
     for (int c = 0; c < kMaxCh; ++c) acc[mp][c] = 0.f;
   }
   const int nkc = (dim + kDC - 1) / kDC, nvc = (vdim + kDC - 1) / kDC;
-  for (int j0 = lo; j0 <= p_last; j0 += kKT) {
+  for (int u0 = 0; u0 < total; u0 += kKT) {
     __syncthreads();  // the previous tile's chunk reads are done (and qs is staged, the first time)
     if (tid < kKT) {
-      const int j = j0 + tid;
-      krow[tid] = j <= p_last ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dc
-                              : -1;
+      const int u = u0 + tid;
+      const int j = u < nk ? u : u - nk + lo;
+      krow[tid] = u < total ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dc
+                            : -1;
     }
-    const int j = j0 + lane;
-    const bool vis = active && j <= pos && j >= my_lo;
+    const int u = u0 + lane;
+    const int j = u < nk ? u : u - nk + lo;
+    const bool vis = active && u < total && j <= pos && (j >= my_lo || j < keep);
     float alpha[MAPS];
 #pragma unroll
     for (int mp = 0; mp < MAPS; ++mp) {
@@ -209,7 +221,9 @@ __global__ __launch_bounds__(64 * kMaxRows) void window_attention_kernel(
           for (int d = 0; d < dn; ++d) sc = __builtin_fmaf(qv[d], kv[d], sc);
         }
       }
-      sc = vis ? sc * scale : -INFINITY;
+      sc *= scale;
+      if (softcap > 0.f) sc = softcap * tanhf(sc * icap);
+      sc = vis ? sc : -INFINITY;
       const float tmax = wave_max(sc);
       float p = 0.f;
       alpha[mp] = 1.f;
@@ -295,7 +309,8 @@ template <typename T, int MAPS>
 void launch_generic(void* out, long out_ld, const void* proj, long proj_ld, const void* cache, int block_size,
                     const int* seq_cu, const int* seq_ctx, const int* seq_bt, int bt_width, int seq0, int seq1,
                     int rows_bound, int tq, int heads, int kv_heads, int dim, int vdim, int gate_off, float scale,
-                    int window, bool sink, float out_scale, float lam, float post, float eps, hipStream_t s) {
+                    int window, bool sink, float out_scale, float lam, float post, float eps, int keep, float softcap,
+                    const float* sink_w, hipStream_t s) {
   const int group = heads / kv_heads;
   auto lds = [&](int rows) {
     return ((size_t)rows * MAPS * dim + kKT * (kDC + 1) + (size_t)rows * MAPS * kKT) * sizeof(float) +
@@ -310,7 +325,8 @@ void launch_generic(void* out, long out_ld, const void* proj, long proj_ld, cons
   dim3 grid(rows_bound / tq + (seq1 - seq0), kv_heads * hchunks), block(64 * nrows);
   window_attention_kernel<T, MAPS><<<grid, block, lds(nrows), s>>>(
       (T*)out, out_ld, (const T*)proj, proj_ld, (const T*)cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0,
-      seq1, tq, hc, hchunks, heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale, lam, post, eps);
+      seq1, tq, hc, hchunks, heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale, lam, post, eps, keep,
+      softcap, sink_w);
 }
 }  // namespace
 
@@ -318,12 +334,12 @@ void launch_window_attention(void* out, long out_ld, const void* proj, long proj
                              const int* seq_cu, const int* seq_ctx, const int* seq_bt, int bt_width, int seq0, int seq1,
                              int rows_bound, int tq, int heads, int kv_heads, int dim, int vdim, int gate_off,
                              float scale, int window, bool sink, float out_scale, int maps, float lam, float post,
-                             float eps, bool f32, hipStream_t s) {
+                             float eps, int keep, float softcap, const float* sink_w, bool f32, hipStream_t s) {
   if (seq1 <= seq0 || rows_bound <= 0) return;
 #define HS_GA(T, M)                                                                                                  \
   launch_generic<T, M>(out, out_ld, proj, proj_ld, cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1,  \
                        rows_bound, tq, heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale, lam, post, \
-                       eps, s)
+                       eps, keep, softcap, sink_w, s)
   if (f32) { if (maps == 2) HS_GA(float, 2); else HS_GA(float, 1); }
   else { if (maps == 2) HS_GA(unsigned short, 2); else HS_GA(unsigned short, 1); }
 #undef HS_GA

@@ -13,11 +13,14 @@
 //   2. S^T = K . Q^T per wave (mfma_f32_16x16x32_bf16, Q operands in registers): lane (c, g) holds
 //      the scores of row c against keys 16 nt + 4 g + i;
 //   3. masked online softmax in fp32 (log2 domain) in registers (a row's scores sit in four lanes); the
-//      sink starts the running (max, sum) at (0, 1);
+//      sink starts the running (max, sum) at (its logit, 1): 0, or a learned number per head; softcap > 0
+//      passes the scaled scores through softcap * tanh(. / softcap) first;
 //   4. O^T += V^T . P^T: the MFMA's k slot (g, e) stands for key 16 (e / 4) + 4 g + e % 4, which is
 //      both where P's registers already are and one 16-byte read of the transposed value tile.
 // Rows with few tokens and many keys (decode) split their keys over grid.z; the runs' unnormalised
 // outputs and (max, sum) are merged by window_attention_reduce.
+// keep > 0: the sequence's first `keep` keys stay visible behind the window. Tiles and runs walk a compacted
+// key index u: the nk kept keys below the workgroup's window first, then the window (key = u - nk + lo).
 //
 // DIFF (differential attention): a query / key head holds two maps [map 1 | map 2]. The wave's two
 // 16-row MFMA tiles are then the two MAPS of the same 16 (token, head) rows: each has its own key
@@ -32,6 +35,10 @@ namespace {
 
 constexpr int kKeys = 32;   // keys per tile
 constexpr int kVLd = 40;    // transposed value tile: row stride in elements (32 keys + pad, 16-byte aligned rows)
+HS_DEVICE float tanh_fast(float x) {  // 1 - 2 / (e^2x + 1); saturates cleanly at both ends
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * 2.88539008177792681f) + 1.f);
+}
+
 constexpr int kNW = 4, kRows = 16 * kNW /* x MT */, kThreads = 64 * kNW, kFT = kThreads / kKeys;
 
 template <int KS> struct KLd { static constexpr int v = KS * 32 + 8; };
@@ -60,7 +67,8 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
     const int* __restrict__ seq_ctx, const int* __restrict__ seq_bt, int bt_width, int seq0, int seq1, int tq, int hc,
     int hchunks, int heads, int kv_heads, int dim, int vdim, int gate_off, float scale, int window, bool sink,
     float out_scale, int part_keys, float* __restrict__ ws_acc, float* __restrict__ ws_ml, int row_base, int ws_rows,
-    float lam, float post, float eps, bool one_row_seqs, bool qvec) {
+    float lam, float post, float eps, bool one_row_seqs, bool qvec, int keep, float softcap,
+    const float* __restrict__ sink_w) {
   static_assert(!DIFF || MT % 2 == 0, "a wave's row tiles come in pairs: the two maps of the same 16 rows");
   constexpr int RT = DIFF ? MT / 2 : MT;   // distinct 16-row tiles per wave; tile mt is rows mt / kMaps, map mt % kMaps
   constexpr int kLd = KLd<KS>::v;
@@ -85,8 +93,12 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
   const int ntok = min(tq, n - tok0);
   const int p_first = ctx - n + tok0, p_last = p_first + ntok - 1;
   const int lo_all = window > 0 ? max(0, p_first - window + 1) : 0;
-  const int lo = lo_all + blockIdx.z * part_keys;
-  const int hi = gridDim.z > 1 ? min(p_last, lo + part_keys - 1) : p_last;
+  const int nk = (window > 0 && keep > 0) ? min(keep, lo_all) : 0;   // kept keys below the workgroup's window
+  const int total = nk + p_last - lo_all + 1;
+  const int lo = blockIdx.z * part_keys;                              // compacted key indices from here on
+  const int hi = gridDim.z > 1 ? min(total - 1, lo + part_keys - 1) : total - 1;
+  auto key_of = [&](int u) { return u < nk ? u : u - nk + lo_all; };
+  const float cap2 = softcap * 1.44269504088896341f, icap = softcap > 0.f ? scale / softcap : 0.f;
   const long Dc = (long)kv_heads * (kMaps * dim + vdim);
   const long koff = (long)kvh * kMaps * dim, voff = (long)kv_heads * kMaps * dim + (long)kvh * vdim;
   const bool first_part = blockIdx.z == 0;
@@ -124,7 +136,7 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
     }
 #pragma unroll
     for (int j = 0; j < NV; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    m_run[mt] = (sink && first_part) ? 0.f : -INFINITY;
+    m_run[mt] = (sink && first_part) ? (sink_w != nullptr ? sink_w[head[mt]] * 1.44269504088896341f : 0.f) : -INFINITY;
     l_run[mt] = (sink && first_part) ? 1.f : 0.f;
   }
   // tile fill: kFT threads per key; key 16 a + 4 gg + b of the tile sits in column 8 gg + 4 a + b of the value tile
@@ -132,9 +144,9 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
   const int vcol = 8 * ((fkey >> 2) & 3) + 4 * (fkey >> 4) + (fkey & 3);
   const int kchunks = dim / 8, vchunks = vdim / 8;
   u16x8 kf[kKF], vf[kVF];
-  auto fetch = [&](int j0) {
-    const int j = j0 + fkey;
-    const bool in = j <= hi;
+  auto fetch = [&](int u0) {
+    const int j = key_of(u0 + fkey);
+    const bool in = u0 + fkey <= hi;
     const long kr = in ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dc : 0;
 #pragma unroll
     for (int i = 0; i < kKF; ++i) {
@@ -201,19 +213,24 @@ __global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
       // (most tiles of a long window) skips the per-key visibility tests.
       float v[8];
       float mx = -INFINITY;
-      const bool whole = sact[mt] && j0 >= s_lo[mt] && j0 + kKeys - 1 <= min(spos[mt], hi);
+      const int ja = key_of(j0), jb = key_of(j0 + kKeys - 1);   // j0: the tile's first compacted index
+      const bool whole = sact[mt] && j0 + kKeys - 1 <= hi && jb - ja == kKeys - 1 && jb <= spos[mt] &&
+                         (ja >= s_lo[mt] || jb < keep);
       if (__all(whole)) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          v[e] = sc[mt][e >> 2][e & 3] * scale2;
+          const float x = sc[mt][e >> 2][e & 3];
+          v[e] = softcap > 0.f ? cap2 * tanh_fast(x * icap) : x * scale2;
           mx = fmaxf(mx, v[e]);
         }
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const int j = j0 + 16 * (e >> 2) + 4 * g + (e & 3);
-          const bool vis = sact[mt] && j <= hi && j <= spos[mt] && j >= s_lo[mt];
-          v[e] = vis ? sc[mt][e >> 2][e & 3] * scale2 : -INFINITY;
+          const int u = j0 + 16 * (e >> 2) + 4 * g + (e & 3);
+          const int j = key_of(u);
+          const bool vis = sact[mt] && u <= hi && j <= spos[mt] && (j >= s_lo[mt] || j < keep);
+          const float x = sc[mt][e >> 2][e & 3];
+          v[e] = vis ? (softcap > 0.f ? cap2 * tanh_fast(x * icap) : x * scale2) : -INFINITY;
           mx = fmaxf(mx, v[e]);
         }
       }
@@ -399,7 +416,8 @@ void launch_mfma(unsigned short* out, long out_ld, const unsigned short* proj, l
                  int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt, int bt_width, int seq0,
                  int seq1, int rows_bound, int heads, int kv_heads, int dim, int vdim, int gate_off, float scale,
                  int window, bool sink, float out_scale, int nparts, int part_keys, float* ws_acc, float* ws_ml,
-                 int row_base, float lam, float post, float eps, hipStream_t s) {
+                 int row_base, float lam, float post, float eps, int keep, float softcap, const float* sink_w,
+                 hipStream_t s) {
   const int group = heads / kv_heads;
   const int rows = kRows * (DIFF ? MT / 2 : MT);
   const int hc = min(group, rows);
@@ -413,7 +431,7 @@ void launch_mfma(unsigned short* out, long out_ld, const unsigned short* proj, l
   window_attention_mfma_kernel<KS, NV, MT, DIFF><<<grid, kThreads, 0, s>>>(
       out, out_ld, proj, proj_ld, cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1, tq, hc, hchunks,
       heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale, part_keys, ws_acc, ws_ml, row_base,
-      rows_bound, lam, post, eps, one_row_seqs, qvec);
+      rows_bound, lam, post, eps, one_row_seqs, qvec, keep, softcap, sink_w);
   if (nparts > 1 && DIFF)
     window_attention_diff_reduce_kernel<<<dim3(rows_bound, heads), 128, 0, s>>>(
         out, out_ld, ws_acc, ws_ml, proj, proj_ld, gate_off, nparts, heads, rows_bound, row_base, vdim, out_scale, lam,
@@ -437,13 +455,15 @@ void launch_window_attention_mfma(void* out, long out_ld, const void* proj, long
                                   int bt_width, int seq0, int seq1, int rows_bound, int heads, int kv_heads, int dim,
                                   int vdim, int gate_off, float scale, int window, bool sink, float out_scale,
                                   int nparts, int part_keys, float* ws_acc, float* ws_ml, int row_base, int maps,
-                                  float lam, float post, float eps, hipStream_t s) {
+                                  float lam, float post, float eps, int keep, float softcap, const float* sink_w,
+                                  hipStream_t s) {
   if (seq1 <= seq0 || rows_bound <= 0) return;
 #define HS_WA(KS, NV, MT, DIFF)                                                                                     \
   launch_mfma<KS, NV, MT, DIFF>((unsigned short*)out, out_ld, (const unsigned short*)proj, proj_ld,                  \
                                 (const unsigned short*)cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0,    \
                                 seq1, rows_bound, heads, kv_heads, dim, vdim, gate_off, scale, window, sink,          \
-                                out_scale, nparts, part_keys, ws_acc, ws_ml, row_base, lam, post, eps, s)
+                                out_scale, nparts, part_keys, ws_acc, ws_ml, row_base, lam, post, eps, keep, softcap,  \
+                                sink_w, s)
   // two row tiles per wave where a prompt portion brings enough rows and the accumulators fit the registers
   const int ks = (dim + 31) / 32, nv = (vdim + 15) / 16;
   const bool wide = nparts == 1 && (long)rows_bound * (heads / kv_heads) >= 128 * (long)(seq1 - seq0);

@@ -41,15 +41,20 @@ HIP_FLAGS = [
 # dense-transformer / sampling / quantisation kernel; "seq" the latent-attention / minGRU / table-MoE
 # kernels of the layer-list decoders (plus the expert alignment of moe.hip); "delta" their window and
 # differential attention, delta-rule and decayed linear-attention recurrences, softmax router and
-# activations. The residual + norm kernels, the expert alignment and the expert GEMMs are linked into
-# both of the latter, so a model of those designs builds only what it runs.
+# activations; "cell" the parallel block with gated sublayer results, the mLSTM matrix memory, PolyNorm and
+# the gate multiply, plus the latent and window attention, router and activations that such a model also
+# runs. Kernel files shared by several libraries are compiled once and linked into each, so a model of
+# those designs builds only what it runs.
 LIBS = {
     "core": ("_C.so", ["kernels/*.hip"], "torch_bindings.cpp"),
     "seq": ("_C_seq.so", ["kernels/seq/group_norm.hip", "kernels/seq/latent_attention*.hip", "kernels/seq/mingru.hip",
                           "kernels/seq/expert_ffn.hip", "kernels/moe.hip"], "seq_bindings.cpp"),
     "delta": ("_C_delta.so", ["kernels/seq/group_norm.hip", "kernels/seq/window_attention*.hip",
                               "kernels/seq/delta_scan.hip", "kernels/seq/router.hip", "kernels/seq/expert_ffn.hip",
-                              "kernels/moe.hip"], "seq_delta_bindings.cpp"),
+                              "kernels/seq/elementwise.hip", "kernels/moe.hip"], "seq_delta_bindings.cpp"),
+    "cell": ("_C_cell.so", ["kernels/seq/gated_block.hip", "kernels/seq/mlstm.hip", "kernels/seq/latent_attention*.hip",
+                            "kernels/seq/window_attention*.hip", "kernels/seq/router.hip", "kernels/seq/expert_ffn.hip",
+                            "kernels/seq/elementwise.hip", "kernels/moe.hip"], "seq_cell_bindings.cpp"),
 }
 
 
@@ -102,7 +107,7 @@ def _compile(src, obj, cmd, want):
 
 def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False, lib: str = "core") -> str:
     """Build one kernel library of ``LIBS`` (gfx950 kernels + torch op registrations):
-    ``core`` = hipserve/_C.so, ``seq`` = hipserve/_C_seq.so, ``delta`` = hipserve/_C_delta.so."""
+    ``core`` = hipserve/_C.so, ``seq`` = hipserve/_C_seq.so, ``delta`` = hipserve/_C_delta.so, ``cell`` = hipserve/_C_cell.so."""
     if not os.path.exists(HIPCC):
         raise RuntimeError(f"hipcc not found at {HIPCC}")
     so_name, patterns, bindings = LIBS[lib]
@@ -226,6 +231,7 @@ def build_all(force: bool = False, jobs: int | None = None, verbose: bool = True
     so = build_kernels(force=force, jobs=jobs, verbose=verbose)
     build_kernels(force=force, jobs=jobs, verbose=verbose, lib="seq")
     build_kernels(force=force, jobs=jobs, verbose=verbose, lib="delta")
+    build_kernels(force=force, jobs=jobs, verbose=verbose, lib="cell")
     return so, rt
 
 

@@ -2,7 +2,7 @@
 
 ``KernelOps`` calls the hand-written gfx950 kernels in ``hipserve/_C.so``
 (``torch.ops.hipserve.*``) and, for the layer-list decoders, ``hipserve/_C_seq.so`` and
-``hipserve/_C_delta.so`` (``torch.ops.hipserve_seq.*``, ``torch.ops.hipserve_delta.*``); each library is loaded at the first use of one of its kernels. ``ReferenceOps`` is the plain-PyTorch oracle used by
+``hipserve/_C_delta.so`` and ``hipserve/_C_cell.so`` (``torch.ops.hipserve_seq.*``, ``torch.ops.hipserve_delta.*``, ``torch.ops.hipserve_cell.*``); each library is loaded at the first use of one of its kernels. ``ReferenceOps`` is the plain-PyTorch oracle used by
 the CPU plumbing engine and by the numerics tests. The choice is made ONCE, when
 an engine is built for a device — never per call. On a GPU device the native
 library is mandatory: a missing/unloadable ``_C.so`` raises instead of silently
@@ -21,10 +21,12 @@ _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 _LIB = os.path.join(_PKG, "_C.so")
 _LIB_SEQ = os.path.join(_PKG, "_C_seq.so")  # the layer-list decoders' kernels (torch.ops.hipserve_seq)
 _LIB_DELTA = os.path.join(_PKG, "_C_delta.so")  # ... window attention / delta rules (torch.ops.hipserve_delta)
+_LIB_CELL = os.path.join(_PKG, "_C_cell.so")  # ... gated parallel blocks, mLSTM, PolyNorm (torch.ops.hipserve_cell)
 _lock = threading.Lock()
 _loaded = False
 _loaded_seq = False
 _loaded_delta = False
+_loaded_cell = False
 
 
 def library_path() -> str:
@@ -80,6 +82,21 @@ def load_delta_library() -> str:
         return _LIB_DELTA
 
 
+def load_cell_library() -> str:
+    """Load hipserve/_C_cell.so into torch.ops (idempotent); built first when it is missing."""
+    global _loaded_cell
+    with _lock:
+        if _loaded_cell:
+            return _LIB_CELL
+        if not os.path.exists(_LIB_CELL):
+            from .._build import build_kernels
+
+            build_kernels(lib="cell")
+        torch.ops.load_library(_LIB_CELL)
+        _loaded_cell = True
+        return _LIB_CELL
+
+
 def core_built() -> bool:
     """True when hipserve/_C.so exists (loaded or not): callers that only PREFER a core kernel ask this, so
     that a model which can do without never triggers the core library's build."""
@@ -103,8 +120,9 @@ class KernelOps:
         self._core = None
         self._seq_ops = None
         self._delta_ops = None
-        # the library whose copy of the shared residual + norm kernel runs ("seq" / "delta"): a model sets it
-        # to the one its mixers load anyway, so it never builds or loads the other
+        self._cell_ops = None
+        # the library whose copy of the shared kernels runs ("seq" / "delta" / "cell"): a model sets it to the one
+        # its mixers load anyway, so it never builds or loads another
         self.norm_library = "seq"
 
     @property
@@ -128,6 +146,23 @@ class KernelOps:
             load_delta_library()
             self._delta_ops = torch.ops.hipserve_delta
         return self._delta_ops
+
+    @property
+    def _cell(self):
+        if self._cell_ops is None:
+            load_cell_library()
+            self._cell_ops = torch.ops.hipserve_cell
+        return self._cell_ops
+
+    @property
+    def _latent_lib(self):
+        """The library whose copy of the latent-attention kernels runs."""
+        return self._cell if self.norm_library == "cell" else self._seq
+
+    @property
+    def _window_lib(self):
+        """The library whose copy of the window attention, router and activation kernels runs."""
+        return self._cell if self.norm_library == "cell" else self._delta
 
     def rmsnorm(self, out, x, w, eps, out8=None):
         """out8: (e4m3 [rows, hidden] uint8, scales fp32 [rows]) per-token FP8 copy of out."""
@@ -221,7 +256,7 @@ class KernelOps:
 
     def latent_prepare(self, cq, cache, proj, positions, slots, q_norm, kv_norm, inv_freq, q_rank, kv_rank,
                        rot_dim, eps):
-        self._seq.latent_prepare(cq, cache, proj, positions, slots, q_norm, kv_norm, inv_freq, q_rank, kv_rank,
+        self._latent_lib.latent_prepare(cq, cache, proj, positions, slots, q_norm, kv_norm, inv_freq, q_rank, kv_rank,
                                  rot_dim, eps)
 
     LATENT_PREFILL_TQ = 4  # tokens per workgroup of a prompt portion (x up to 4 heads = 16 waves)
@@ -232,7 +267,7 @@ class KernelOps:
     def latent_query_in_place(self, dtype, kv_rank, rot_dim) -> bool:
         """True when ``latent_attention`` wants the absorbed queries as bf16 rows of the cached width
         ([heads, T, kv_rank + rot_dim], the rotary part left for it to fill) instead of fp32 [heads, T, kv_rank]."""
-        return dtype == torch.bfloat16 and self.LATENT_MFMA and bool(self._seq.latent_attention_mfma_ok(kv_rank, rot_dim))
+        return dtype == torch.bfloat16 and self.LATENT_MFMA and bool(self._latent_lib.latent_attention_mfma_ok(kv_rank, rot_dim))
 
     def latent_attention(self, o_lat, q_abs, q, proj, cache, meta, inv_freq, heads, dim, rot_dim, kv_rank,
                          gate_off, scale, window):
@@ -241,7 +276,7 @@ class KernelOps:
         nseq = meta.seq_ctx.shape[0]
         nd = meta.num_decode
         npf, Tp = nseq - nd, meta.num_prefill_tokens
-        if (q.dtype == torch.bfloat16 and self.LATENT_MFMA and self._seq.latent_attention_mfma_ok(kv_rank, rot_dim)):
+        if (q.dtype == torch.bfloat16 and self.LATENT_MFMA and self._latent_lib.latent_attention_mfma_ok(kv_rank, rot_dim)):
             # bf16: the matrix-core kernel; decode rows split their keys into runs merged by a reduce kernel
             if q_abs.dtype == torch.bfloat16:  # the absorption GEMM wrote the rows in place (latent_query_in_place)
                 qc, q_abs = q_abs, None
@@ -249,7 +284,7 @@ class KernelOps:
                 qc = torch.empty(heads, q.shape[0], kv_rank + rot_dim, device=q.device, dtype=q.dtype)
             fill = True
             if npf:
-                self._seq.latent_attention_mfma(o_lat, qc, q_abs, q, proj, meta.positions, cache, meta.seq_cu,
+                self._latent_lib.latent_attention_mfma(o_lat, qc, q_abs, q, proj, meta.positions, cache, meta.seq_cu,
                                                 meta.seq_ctx, meta.seq_bt, 0, npf, Tp, inv_freq, heads, dim, rot_dim,
                                                 kv_rank, gate_off, scale, window, 1, 0, None, None, 0, fill)
                 fill = False
@@ -263,13 +298,13 @@ class KernelOps:
                 if nparts > 1:
                     ws_acc = torch.empty(nparts, heads, nd, kv_rank, device=q.device, dtype=torch.float32)
                     ws_ml = torch.empty(nparts, heads, nd, 2, device=q.device, dtype=torch.float32)
-                self._seq.latent_attention_mfma(o_lat, qc, q_abs, q, proj, meta.positions, cache, meta.seq_cu,
+                self._latent_lib.latent_attention_mfma(o_lat, qc, q_abs, q, proj, meta.positions, cache, meta.seq_cu,
                                                 meta.seq_ctx, meta.seq_bt, npf, nseq, nd, inv_freq, heads, dim, rot_dim,
                                                 kv_rank, gate_off, scale, window, nparts, part, ws_acc, ws_ml, Tp, fill)
             return
         for s0, s1, rows, tq in ((0, npf, Tp, self.LATENT_PREFILL_TQ), (npf, nseq, nd, 1)):
             if s1 > s0:
-                self._seq.latent_attention(o_lat, q_abs, q, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt,
+                self._latent_lib.latent_attention(o_lat, q_abs, q, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt,
                                            s0, s1, rows, tq, inv_freq, heads, dim, rot_dim, kv_rank, gate_off,
                                            scale, window)
 
@@ -279,7 +314,7 @@ class KernelOps:
     def attn_prepare(self, proj, cache, meta, inv_freq, sp, q_norm, k_norm, eps):
         mode = 1 if sp.qk_norm else 2 if sp.head_norm else 0
         own_kv = sp.kv_from is None   # else the layer reads another layer's cache: only q is prepared
-        self._delta.attn_prepare(proj, cache if own_kv else None, meta.positions, meta.slot_mapping, inv_freq, sp.heads,
+        self._window_lib.attn_prepare(proj, cache if own_kv else None, meta.positions, meta.slot_mapping, inv_freq, sp.heads,
                                  sp.kv_heads, sp.maps, sp.dim, sp.vdim, q_norm if mode else None,
                                  k_norm if mode and own_kv else None, mode, sp.v_norm, eps)
 
@@ -288,23 +323,26 @@ class KernelOps:
     WINDOW_MFMA = os.environ.get("HIPSERVE_WINDOW_MFMA", "1") != "0"
     WINDOW_DECODE_RUN = 128  # keys per run of a decode row (a multiple of 32)
 
-    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0, lam=0.0, eps=0.0):
+    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0, lam=0.0, eps=0.0, sink_w=None):
         """Prompt portions (the step's first sequences) run several tokens per workgroup, decode
         rows one token per workgroup. Two maps per head (``sp.maps`` = 2): ``lam`` weighs the second
-        map, the head output is divided by its root mean square (``eps``) and scaled by 1 - ``sp.diff``."""
+        map, the head output is divided by its root mean square (``eps``) and scaled by 1 - ``sp.diff``.
+        ``sink_w``: fp32 [heads] learned sink logits (None: 0)."""
         nseq = meta.seq_ctx.shape[0]
         nd = meta.num_decode
         npf, Tp = nseq - nd, meta.num_prefill_tokens
-        diff = (sp.maps, lam, 1.0 - sp.diff, eps)
+        diff = (sp.maps, lam, 1.0 - sp.diff, eps, sp.keep_first, sp.softcap, sink_w)
         if (proj.dtype == torch.bfloat16 and self.WINDOW_MFMA
-                and self._delta.window_attention_mfma_ok(sp.dim, sp.vdim, out.stride(0), out.storage_offset(), sp.maps)):
+                and self._window_lib.window_attention_mfma_ok(sp.dim, sp.vdim, out.stride(0), out.storage_offset(), sp.maps)):
             # bf16: the matrix-core kernel; decode rows split their keys into runs merged by a reduce kernel
             args = (sp.heads, sp.kv_heads, sp.dim, sp.vdim, gate_off, sp.scale, sp.window, sp.sink, out_scale)
             if npf:
-                self._delta.window_attention_mfma(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, 0, npf, Tp,
+                self._window_lib.window_attention_mfma(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, 0, npf, Tp,
                                                 *args, 1, 0, None, None, 0, *diff)
             if nd:
-                span = min(sp.window, meta.max_ctx or sp.window) if sp.window > 0 else meta.max_ctx
+                # keys a row can see: its window and the kept first keys behind it
+                reach = sp.window + sp.keep_first
+                span = min(reach, meta.max_ctx or reach) if sp.window > 0 else meta.max_ctx
                 part = self.WINDOW_DECODE_RUN
                 if span >= 16 * part:   # long runs of keys: fewer, longer runs per row (measured at 2k and 8k keys)
                     part *= 2
@@ -315,12 +353,12 @@ class KernelOps:
                 if nparts > 1:
                     ws_acc = torch.empty(nparts, sp.heads * sp.maps, nd, sp.vdim, device=proj.device, dtype=torch.float32)
                     ws_ml = torch.empty(nparts, sp.heads * sp.maps, nd, 2, device=proj.device, dtype=torch.float32)
-                self._delta.window_attention_mfma(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, npf, nseq, nd,
+                self._window_lib.window_attention_mfma(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, npf, nseq, nd,
                                                 *args, nparts, part, ws_acc, ws_ml, Tp, *diff)
             return
         for s0, s1, rows, tq in ((0, npf, Tp, self.WINDOW_PREFILL_TQ), (npf, nseq, nd, 1)):
             if s1 > s0:
-                self._delta.window_attention(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, s0, s1, rows, tq,
+                self._window_lib.window_attention(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, s0, s1, rows, tq,
                                            sp.heads, sp.kv_heads, sp.dim, sp.vdim, gate_off, sp.scale, sp.window,
                                            sp.sink, out_scale, *diff)
 
@@ -339,7 +377,7 @@ class KernelOps:
     ACTIVATIONS = {"tanh": 0, "xielu": 1, "relu2": 2, "silu_mul": 3}
 
     def activation(self, out, x, kind, c0=0.0, c1=0.0):
-        self._delta.activation(out, x, self.ACTIVATIONS[kind], c0, c1)
+        self._window_lib.activation(out, x, self.ACTIVATIONS[kind], c0, c1)
         return out
 
     def add_normed(self, out, residual, y, w, eps, moe=None):
@@ -366,16 +404,42 @@ class KernelOps:
 
     ROUTER_MAX_OUTPUTS = 256
 
-    def route_topk(self, ids, wts, logits, correction, top, scale, E):
-        if logits.shape[1] > self.ROUTER_MAX_OUTPUTS:   # more router outputs than a wave holds: device-side torch ops
-            ref.route_topk(ids, wts, logits, correction, top, scale, E)
+    def route_topk(self, ids, wts, logits, correction, top, scale, E, groups=1, keep_groups=1, renorm=False):
+        if logits.shape[1] > self.ROUTER_MAX_OUTPUTS or groups > 64:
+            # more router outputs than a wave holds: device-side torch ops
+            ref.route_topk(ids, wts, logits, correction, top, scale, E, groups, keep_groups, renorm)
             return
-        self._delta.route_topk(ids, wts, logits.contiguous(), correction, top, scale, E)
+        self._window_lib.route_topk(ids, wts, logits.contiguous(), correction, top, scale, E, groups, keep_groups, renorm)
+
+    # ---- parallel blocks with gated sublayer results, mLSTM, PolyNorm (csrc/kernels/seq/gated_block.hip, mlstm.hip,
+    # elementwise.hip)
+    def gated_add_norms(self, out1, out2, residual, w1, w2, eps, first=None, second=None):
+        """``first`` / ``second``: (y, g, b) of a sublayer, y its result rows or, for a mixture of experts,
+        (ye, pair_slot, wts, shared)."""
+        y1, g1, b1 = first if first is not None else (None, None, None)
+        y2, g2, b2 = second if second is not None else (None, None, None)
+        parts = (None, None, None, None)
+        if isinstance(y2, tuple):
+            parts, y2 = y2, None
+        self._cell.gated_add_norms(out1, out2, residual, w1, w2, eps, y1, g1, b1, y2, g2, b2, *parts)
+
+    def polynorm(self, out, x, coef, eps):
+        self._cell.polynorm(out, x, coef, eps)
+        return out
+
+    def gate_mul(self, out, x, gate):
+        self._cell.gate_mul(out, x, gate)
+        return out
+
+    def mlstm(self, out, state, proj, gates, b_if, norm_w, sp, eps, meta):
+        scratch = torch.empty(proj.shape[0] * sp.heads * (sp.vdim + 5), device=proj.device, dtype=torch.float32)
+        self._cell.mlstm(out, state[0], state[1], state[2], proj, gates, b_if, norm_w, meta.seq_cu, meta.seq_ctx,
+                         meta.seq_state, scratch, sp.heads, sp.dim, sp.vdim, sp.gate_cap, eps, meta.max_q == 1)
 
     @property
     def _moe_lib(self):
         """The library whose copy of the expert alignment and expert GEMMs runs (the one the model loads anyway)."""
-        return self._delta if self.norm_library == "delta" else self._seq
+        return {"delta": self._delta, "cell": self._cell}.get(self.norm_library) or self._seq
 
     def moe_align(self, experts, E, tile, slots, tile_expert, pair_slot):
         if E <= 128:
