@@ -1294,3 +1294,33 @@ PRESETS.update({
                                    dict(heads=8, kv_heads=2, dim=32, vdim=64, scale=32 ** -0.5, diff=0.5), 1536,
                                    dict(experts=8, top=2, ff=256, identity=2, scale=1.0, shared_ff=512), "wasw"),
 })
+
+
+def _mini_topezen(name, H, V, latent, mlstm, attn, ff, moe, order, embed_scale=4.0):
+    """order: 'l' latent attention + dense feed-forward, 'm' matrix memory + routed experts, 'a' capped window
+    attention with a learned sink + routed experts, 'n' matrix memory without a feed-forward."""
+    f, e = DenseFFSpec(ff, "polynorm"), RoutedMoESpec(renorm=True, **moe)
+    spec = {"l": HybridLayerSpec(LatentAttentionSpec(interleaved=True, gate="channel", **latent), f),
+            "m": HybridLayerSpec(MLstmSpec(**mlstm), e),
+            "a": HybridLayerSpec(WindowAttentionSpec(head_norm=True, sink=True, sink_weights=True, **attn), e),
+            "n": HybridLayerSpec(MLstmSpec(**mlstm), None)}
+    return TopezenConfig(name=name, hidden_size=H, vocab_size=V, layers=tuple(spec[c] for c in order),
+                         embed_scale=embed_scale, eos_token_id=(2,), bos_token_id=1)
+
+
+PRESETS.update({
+    # CPU plumbing size
+    "tiny-topezen": _mini_topezen("tiny-topezen", 64, 320,
+                                  dict(heads=3, dim=16, rot_dim=8, vdim=24, q_rank=40, kv_rank=32, scale=24 ** -0.5),
+                                  dict(heads=2, dim=16, vdim=24, gate_cap=10.0),
+                                  dict(heads=4, kv_heads=2, dim=16, vdim=8, scale=0.25, window=24, keep_first=5, softcap=30.0),
+                                  96, dict(experts=6, top=2, ff=24, shared_ff=40, groups=3, keep_groups=2), "lmanl"),
+    # GPU-test size
+    "small-topezen": _mini_topezen("small-topezen", 512, 1024,
+                                   dict(heads=8, dim=64, rot_dim=32, vdim=64, q_rank=192, kv_rank=128, scale=96 ** -0.5,
+                                        rot_base=50000.0),
+                                   dict(heads=4, dim=64, vdim=128, gate_cap=15.0),
+                                   dict(heads=8, kv_heads=2, dim=64, vdim=64, scale=0.125, window=160, keep_first=16,
+                                        softcap=50.0),
+                                   1536, dict(experts=8, top=2, ff=256, shared_ff=512, groups=4, keep_groups=2), "lmam"),
+})

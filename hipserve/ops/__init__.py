@@ -439,7 +439,9 @@ class KernelOps:
     @property
     def _moe_lib(self):
         """The library whose copy of the expert alignment and expert GEMMs runs (the one the model loads anyway)."""
-        return {"delta": self._delta, "cell": self._cell}.get(self.norm_library) or self._seq
+        if self.norm_library == "cell":
+            return self._cell
+        return self._delta if self.norm_library == "delta" else self._seq
 
     def moe_align(self, experts, E, tile, slots, tile_expert, pair_slot):
         if E <= 128:

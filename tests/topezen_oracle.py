@@ -195,3 +195,101 @@ def forward(cfg: dict, tensors: dict, tokens, states=None, return_layers: bool =
     if return_layers:
         return logits, torch.stack(after), new_states
     return logits
+
+
+# ------------------------------------------------------------------ small configs and random weights
+def latent_layer(heads=3, dim=8, rot_dim=4, vdim=6, q_rank=10, kv_rank=12, scale=None, base=10000.0, mlp=None):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+         "scale": scale or (dim + rot_dim) ** -0.5, "rot": {"base": base, "dims": rot_dim}}
+    return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+
+def mlstm_layer(heads=2, dim=8, vdim=12, gate_cap=10.0, mlp=None):
+    return {"type": "mlstm", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "gate_cap": gate_cap}, "mlp": mlp}
+
+
+def attn_layer(heads=4, kv_heads=2, dim=8, vdim=12, scale=None, softcap=15.0, size=11, keep_first=3, mlp=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale or dim ** -0.5,
+         "softcap": softcap, "mask": {"size": size, "keep_first": keep_first}}
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def dense(ff=40):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts=6, top=2, ff=12, count=3, keep=2, shared=20):
+    f = {"kind": "moe", "expert": {"ff": ff},
+         "router": {"experts": experts, "top": top, "groups": {"count": count, "keep": keep}}}
+    if shared:
+        f["shared"] = {"ff": shared}
+    return f
+
+
+def make_config(layers, width=32, vocab=96, eps=1e-5, scale=3.0):
+    return {"architecture": "Topezen", "embedding": {"scale": scale}, "layers": layers, "norm": {"eps": eps},
+            "vocab": vocab, "width": width}
+
+
+def make_weights(cfg, seed=0, gain=1.0):
+    """Random checkpoint tensors (values representable in bf16) under the design's names."""
+    g = torch.Generator().manual_seed(seed)
+    Wd, V = cfg["width"], cfg["vocab"]
+
+    def rnd(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g) * std).bfloat16().float()
+
+    def lin(o, i):
+        return rnd(o, i, std=gain / math.sqrt(i))
+
+    W = {"embed": rnd(V, Wd, std=1.0 / cfg["embedding"]["scale"]), "head": lin(V, Wd) * 3, "final.norm": (1 + rnd(1, std=0.2)).reshape(())}
+    for i, l in enumerate(cfg["layers"]):
+        p, m, f = f"l{i}.mix.", l["mixer"], l["mlp"]
+        W[f"l{i}.norm1"] = (1 + rnd(1, std=0.2)).reshape(())
+        W[f"l{i}.rg1"], W[f"l{i}.rg1.b"] = lin(Wd, Wd) * 2, rnd(Wd, std=0.5)
+        if l["type"] == "latent_attention":
+            H, d, r, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+            W[p + "dq"], W[p + "dq.norm"] = lin(m["q_rank"], Wd) * 2, 1 + rnd(m["q_rank"], std=0.2)
+            W[p + "uq"] = lin(H * (d + r), m["q_rank"]) * 2
+            W[p + "dkv"], W[p + "dkv.norm"] = lin(m["kv_rank"] + r, Wd) * 2, 1 + rnd(m["kv_rank"], std=0.2)
+            W[p + "uk"], W[p + "uv"] = lin(H * d, m["kv_rank"]) * 2, lin(H * dv, m["kv_rank"]) * 2
+            W[p + "g"], W[p + "o"] = lin(H * dv, Wd) * 2, lin(Wd, H * dv)
+        elif l["type"] == "mlstm":
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            W[p + "q"], W[p + "k"], W[p + "v"] = lin(H * d, Wd) * 2, lin(H * d, Wd) * 2, lin(H * dv, Wd) * 2
+            W[p + "i"], W[p + "i.b"] = lin(H, Wd) * 3, rnd(H)
+            W[p + "f"], W[p + "f.b"] = lin(H, Wd) * 3, rnd(H) + 2.0
+            W[p + "g"], W[p + "norm"], W[p + "o"] = lin(H * dv, Wd) * 2, 1 + rnd(H * dv, std=0.2), lin(Wd, H * dv)
+        else:
+            H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            W[p + "q"], W[p + "q.norm"] = lin(H * d, Wd) * 2, 1 + rnd(d, std=0.3)
+            W[p + "k"], W[p + "k.norm"] = lin(G * d, Wd) * 2, 1 + rnd(d, std=0.3)
+            W[p + "v"], W[p + "sink"], W[p + "o"] = lin(G * dv, Wd) * 2, rnd(H), lin(Wd, H * dv)
+        if f is None:
+            continue
+        p = f"l{i}.mlp."
+        W[f"l{i}.norm2"] = (1 + rnd(1, std=0.2)).reshape(())
+        W[f"l{i}.rg2"], W[f"l{i}.rg2.b"] = lin(Wd, Wd) * 2, rnd(Wd, std=0.5)
+        if f["kind"] == "dense":
+            W[p + "up"], W[p + "down"], W[p + "act"] = lin(f["ff"], Wd) * 2, lin(Wd, f["ff"]), rnd(4, std=0.7)
+        else:
+            n = f["router"]["experts"]
+            W[p + "router"], W[p + "correction"] = lin(n, Wd) * 3, rnd(n, std=0.1)
+            names = [f"e{e}." for e in range(n)] + (["shared."] if f.get("shared") else [])
+            for e in names:
+                ff = f["shared"]["ff"] if e == "shared." else f["expert"]["ff"]
+                W[p + e + "gate"], W[p + e + "up"], W[p + e + "down"] = lin(ff, Wd) * 2, lin(ff, Wd) * 2, lin(Wd, ff)
+    return {k: v.bfloat16().float() for k, v in W.items()}
+
+
+def save_checkpoint(path, cfg, W):
+    import json
+    import os
+
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.bfloat16().contiguous() for k, v in W.items()}, os.path.join(path, "model.safetensors"))
+    return path
