@@ -126,8 +126,8 @@ def test_matrix_memory_alone(target, shape):
         assert rel_err(got, want) < TOL[target[1]]
         # the slot holds the state scaled by exp(-m): compare what does not depend on the path of m
         m = state[2][1].double().cpu()
-        assert torch.allclose(state[0][1].double().cpu() * torch.exp(m - st[2])[:, None, None], st[0],
-                              rtol=5e-2 if target[1] == "bfloat16" else 1e-3, atol=1e-3)
+        held = state[0][1].double().cpu() * torch.exp(m - st[2])[:, None, None]
+        assert float((held - st[0]).norm() / st[0].norm()) < (2e-2 if target[1] == "bfloat16" else 1e-4)
         assert float(state[0][0].min()) == 7.0 and float(state[2][2].max()) == 7.0   # the other slots are untouched
 
 
@@ -162,7 +162,8 @@ def test_matrix_memory_long_and_tiny_values(target):
     h = rows(300, 24, 5).double()
     want, _ = O.mlstm(h, d64(W), l["mixer"], EPS)
     got, _ = run_mixer(l, W, h.float(), target, [(0, 130), (130, 131), (131, 195), (195, 300)], total=304)
-    assert rel_err(got, want) < TOL[target[1]]
+    # bf16: the rows as a whole (the worst single row of 300 lands on an output that is small all over)
+    check_all({("s", p): r for p, r in enumerate(got.float().cpu())}, "s", want, TOL[target[1]])
 
 
 @pytest.mark.parametrize("target", TARGETS)
@@ -495,6 +496,18 @@ def test_config_reader():
         TopezenConfig.from_dict(bad)
 
 
+def assert_greedy(cfg, W, prompt, out, slack, flips=0):
+    """Every generated token is an argmax (within ``slack``) of the oracle's logits over the tokens before it. In
+    bf16 up to ``flips`` positions may differ: among a hundred routed tokens of a tiny random model some have two
+    experts whose choice scores differ by 1e-4, which the rounding of the router's input decides the other way,
+    and another expert moves the logits by far more than rounding does. The tokens after it are checked against
+    the oracle on the engine's own continuation, so a lost state or key would still show on all of them."""
+    lg = O.forward(cfg, W, prompt + out)
+    bad = [(k, t, int(lg[len(prompt) + k - 1].argmax())) for k, t in enumerate(out)
+           if lg[len(prompt) + k - 1][t] < lg[len(prompt) + k - 1].max() - slack]
+    assert len(bad) <= flips, bad
+
+
 @pytest.mark.parametrize("target", TARGETS)
 def test_greedy_generation_through_the_scheduler(tmp_path, target):
     """LLMEngine.generate: the scheduler's own chunked prefill (a 24-token budget), batching of three
@@ -514,10 +527,7 @@ def test_greedy_generation_through_the_scheduler(tmp_path, target):
     slack = 1e-3 if target == CPU else (0.07 if target[1] == "float32" else 0.15)
     for p, (out, _text, reason) in zip(prompts, res):
         assert len(out) == 12 and reason == "length"
-        lg = O.forward(cfg, W, p + out)
-        for k, t in enumerate(out):
-            row = lg[len(p) + k - 1]
-            assert row[t] >= row.max() - slack, (k, t, int(row.argmax()))
+        assert_greedy(cfg, W, p, out, slack, flips=1 if target[1] == "bfloat16" else 0)
     assert eng.states.num_free() == 4 and eng.blocks.num_free() == eng.blocks.num_blocks
 
 
@@ -540,10 +550,7 @@ def test_graph_decode_matches_eager_gpu(tmp_path):
         if not eager:
             assert eng.runner.stats["graph_steps"] > 0
     for p, out in zip(prompts, outs[1]):
-        lg = O.forward(cfg, W, p + out)
-        for k, t in enumerate(out):
-            row = lg[len(p) + k - 1]
-            assert row[t] >= row.max() - 0.3, (k, t, int(row.argmax()))
+        assert_greedy(cfg, W, p, out, 0.3, flips=2)
     same = sum(a == b for a, b in zip(outs[0], outs[1]))
     assert same >= len(prompts) - 1, (outs[0], outs[1])  # bf16 near-ties may flip one continuation
 
