@@ -81,7 +81,7 @@ def parse():
                     help="instead of the headline benchmark: prefill / decode tok/s of a layer-list decoder "
                          "beside the closest family at equal size (hipserve/bench/layer_compare.py)")
     ap.add_argument("--layer-sizes", default="", help="with --layer-compare: sizes, comma separated (default: all)")
-    ap.add_argument("--layer-models", default="", help="with --layer-compare: any of kesirax, mixtral, fikizen, dense, kemavik (default: kesirax,mixtral)")
+    ap.add_argument("--layer-models", default="", help="with --layer-compare: any of kesirax, mixtral, fikizen, dense, kemavik, topezen (default: kesirax,mixtral)")
     ap.add_argument("--layer-batch", type=int, default=16)
     ap.add_argument("--layer-prompt", type=int, default=2048)
     ap.add_argument("--layer-new", type=int, default=64)

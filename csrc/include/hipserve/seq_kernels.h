@@ -157,7 +157,7 @@ void launch_gated_add_norms(void* out1, void* out2, float* residual, const float
 
 // mLSTM matrix memory over state slots (mlstm.hip): proj rows = [q | k | v | gate | ...], gates fp32 [T, 2 heads] =
 // [input | forget] pre-activations, b_if their biases, S [slots, heads, dim, vdim], N [slots, heads, dim],
-// M [slots, heads]; scratch: T * heads * (vdim + 5) floats. one_row_seqs: every sequence brings one row.
+// M [slots, heads]; scratch: T * heads * (2 dim + 2 vdim + 6) floats. one_row_seqs: every sequence brings one row.
 int mlstm_max_dim();
 void launch_mlstm(void* out, float* S, float* N, float* M, const void* proj, long ld, const float* gates,
                   const float* b_if, const float* norm_w, const int* seq_cu, const int* seq_ctx, const int* seq_state,

@@ -97,6 +97,48 @@ __global__ __launch_bounds__(256) void polynorm_kernel(T* __restrict__ out, long
   }
 }
 
+// bf16 rows whose length, strides and base addresses are multiples of 8 elements: NV 16-byte vectors per thread
+// (rows up to 2048 NV wide), read once.
+template <int NV>
+__global__ __launch_bounds__(256) void polynorm_vec_kernel(unsigned short* __restrict__ out, long out_ld,
+                                                           const unsigned short* __restrict__ x, long x_ld, int cols,
+                                                           const float* __restrict__ coef, float eps) {
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x;
+  u16x8 z[NV];
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = 8 * (tid + 256 * i);
+    z[i] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if (c < cols) z[i] = *reinterpret_cast<const u16x8*>(x + t * x_ld + c);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = bf16_to_f32(z[i][e]), q = v * v;
+      s2 += q; s4 += q * q; s6 += q * q * q;
+    }
+  }
+  s2 = block_sum(s2, red);
+  s4 = block_sum(s4, red);
+  s6 = block_sum(s6, red);
+  const float n = (float)cols;
+  const float a = coef[0] / sqrtf(s2 / n + eps), b = coef[1] / sqrtf(s4 / n + eps), c3 = coef[2] / sqrtf(s6 / n + eps);
+  const float e0 = coef[3];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = 8 * (tid + 256 * i);
+    if (c >= cols) continue;
+    u16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = bf16_to_f32(z[i][e]);
+      r[e] = f32_to_bf16(((c3 * v + b) * v + a) * v + e0);
+    }
+    *reinterpret_cast<u16x8*>(out + t * out_ld + c) = r;
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void gate_mul_kernel(T* __restrict__ out, const T* __restrict__ x,
                                                        const T* __restrict__ gate, long gate_ld, int T_rows, int d,
@@ -127,6 +169,15 @@ void launch_activation(void* out, long out_ld, const void* x, long x_ld, int row
 void launch_polynorm(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, const float* coef,
                      float eps, bool f32, hipStream_t s) {
   if (rows <= 0 || cols <= 0) return;
+  if (!f32 && cols % 8 == 0 && out_ld % 8 == 0 && x_ld % 8 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)x % 16 == 0 &&
+      cols <= 2048 * 4) {
+    auto o = (unsigned short*)out;
+    auto in = (const unsigned short*)x;
+    if (cols <= 2048) polynorm_vec_kernel<1><<<rows, 256, 0, s>>>(o, out_ld, in, x_ld, cols, coef, eps);
+    else if (cols <= 4096) polynorm_vec_kernel<2><<<rows, 256, 0, s>>>(o, out_ld, in, x_ld, cols, coef, eps);
+    else polynorm_vec_kernel<4><<<rows, 256, 0, s>>>(o, out_ld, in, x_ld, cols, coef, eps);
+    return;
+  }
   const bool reg = cols <= 256 * kPolyPer;
 #define HS_PN(T, R) polynorm_kernel<T, R><<<rows, 256, 0, s>>>((T*)out, out_ld, (const T*)x, x_ld, cols, coef, eps)
   if (f32) { if (reg) HS_PN(float, true); else HS_PN(float, false); }

@@ -7,7 +7,10 @@
 //   out = o / sqrt(mean_head(o^2) + eps) * w * sigmoid(gate)
 // A step that starts at position 0 starts from S = 0, n = 0, m = 0.
 //
-// Prompt portions run three kernels:
+// Prompt portions run four kernels:
+//   mlstm_stage  one workgroup per token: q (scaled), k and v of every head as dense fp32 rows, the value row one
+//                element longer with a 1 at its end (the normaliser's value), so the scan stages everything with
+//                contiguous 4-byte loads whatever the element type and the row stride of the projection
 //   mlstm_gates  one wave per (sequence, head): the gates of 64 tokens at a time and the running maximum by a
 //                wave scan in the (max, +) semiring (m' = max(m + F, I) composes as F = F1 + F2,
 //                I = max(I1 + F2, I2)); writes a, b and exp(-m) per token and the last m into the slot.
@@ -65,6 +68,30 @@ __global__ __launch_bounds__(64) void mlstm_gates_kernel(f32x4* __restrict__ scr
   if (lane == 0) *mp = carry;
 }
 
+// qk[t, h] = [q * qscale (dim) | k (dim)], vv[t, h] = [v (vdim) | 1]
+template <typename T>
+__global__ __launch_bounds__(256) void mlstm_stage_kernel(float* __restrict__ qk, float* __restrict__ vv,
+                                                         const T* __restrict__ proj, long ld, int heads, int dim,
+                                                         int vdim, float qscale) {
+  const long t = blockIdx.x;
+  const T* row = proj + t * ld;
+  const int nqk = heads * dim, nv = heads * vdim;
+  for (int e = threadIdx.x; e < nqk; e += 256) {
+    const int h = e / dim, i = e - h * dim;
+    float* dst = qk + (t * heads + h) * 2 * dim;
+    dst[i] = ldf<T>(row, e) * qscale;
+    dst[dim + i] = ldf<T>(row, nqk + e);
+  }
+  for (int e = threadIdx.x; e < nv + heads; e += 256) {
+    if (e < nv) {
+      const int h = e / vdim, c = e - h * vdim;
+      vv[(t * heads + h) * (vdim + 1) + c] = ldf<T>(row, 2L * nqk + e);
+    } else {
+      vv[(t * heads + (e - nv)) * (vdim + 1) + vdim] = 1.f;
+    }
+  }
+}
+
 constexpr int kTB = 8;     // tokens staged at a time
 constexpr int kSeg = 16;   // lanes that share a state column (one DPP row)
 constexpr int kScanThreads = 256;
@@ -79,11 +106,11 @@ HS_DEVICE float row_sum(float v) {
 
 // grid (heads, ceil((vdim + 1) / kCols), sequences). Column c < vdim is S[:, c]; column vdim is the normaliser.
 // o [T, heads, vdim + 1]: the unnormalised read-outs, the last one n . q.
-template <typename T, int DS>
+template <int DS>
 __global__ __launch_bounds__(kScanThreads) void mlstm_scan_kernel(
-    float* __restrict__ o, float* __restrict__ S, float* __restrict__ N, const T* __restrict__ proj, long ld,
-    const f32x4* __restrict__ scr, const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx,
-    const int* __restrict__ seq_state, int heads, int dim, int vdim, float qscale) {
+    float* __restrict__ o, float* __restrict__ S, float* __restrict__ N, const float* __restrict__ qk,
+    const float* __restrict__ vv, const f32x4* __restrict__ scr, const int* __restrict__ seq_cu,
+    const int* __restrict__ seq_ctx, const int* __restrict__ seq_state, int heads, int dim, int vdim) {
   constexpr int DP = kSeg * DS;
   __shared__ __attribute__((aligned(16))) float sq[kTB][DP], sk[kTB][DP];
   __shared__ float sab[kTB][2];
@@ -106,9 +133,8 @@ __global__ __launch_bounds__(kScanThreads) void mlstm_scan_kernel(
       else if (is_n) st[i] = Np[k0 + i];
     }
   }
-  const long qoff = (long)h * dim, koff = (long)heads * dim + (long)h * dim;
-  const long voff = 2L * heads * dim + (long)h * vdim + c;
   const int ow = vdim + 1;
+  const bool has_col = c <= vdim;
   constexpr int kLd = (kTB * DP + kScanThreads - 1) / kScanThreads;
   float rq[kLd], rk[kLd], rv[kTB], rab = 0.f;
   auto fetch = [&](int t0) {
@@ -117,10 +143,10 @@ __global__ __launch_bounds__(kScanThreads) void mlstm_scan_kernel(
     for (int it = 0; it < kLd; ++it) {
       const int i = it * kScanThreads + tid;
       const int tt = i / DP, k = i % DP;
-      const T* row = proj + (long)(r0 + t0 + tt) * ld;
+      const float* row = qk + ((long)(r0 + t0 + tt) * heads + h) * 2 * dim;
       const bool in = tt < nt && k < dim;
-      rq[it] = in ? ldf<T>(row, qoff + k) * qscale : 0.f;
-      rk[it] = in ? ldf<T>(row, koff + k) : 0.f;
+      rq[it] = in ? row[k] : 0.f;
+      rk[it] = in ? row[dim + k] : 0.f;
     }
     if (tid < 2 * nt) {
       const f32x4 g = scr[(long)(r0 + t0 + (tid >> 1)) * heads + h];
@@ -128,7 +154,7 @@ __global__ __launch_bounds__(kScanThreads) void mlstm_scan_kernel(
     }
 #pragma unroll
     for (int tt = 0; tt < kTB; ++tt)
-      rv[tt] = is_n ? 1.f : (tt < nt && is_s) ? ldf<T>(proj, (long)(r0 + t0 + tt) * ld + voff) : 0.f;
+      rv[tt] = (tt < nt && has_col) ? vv[((long)(r0 + t0 + tt) * heads + h) * ow + c] : 0.f;
   };
   float* po = o + ((long)r0 * heads + h) * ow + c;
   fetch(0);
@@ -196,9 +222,12 @@ __global__ __launch_bounds__(256) void mlstm_out_kernel(T* __restrict__ out, con
 
 constexpr int kStepCols = 4;   // state columns per thread of the one-row kernel (vdim <= 4 * 256)
 
-// grid (heads, sequences), 256 threads; sequence s brings the one row seq_cu[s]. Dynamic LDS: q, k [dim] each.
+// grid (heads, sequences), 256 G threads (G = 1, 2 or 4 row groups); sequence s brings the one row seq_cu[s].
+// Thread (g, c) walks its quarter of the key channels of state column c (+ 256 per pass), eight rows' loads in
+// flight before their updates are stored; the groups' partial read-outs meet in LDS. Dynamic LDS: q, k [dim]
+// each, then (G - 1) x 256 partial sums.
 template <typename T>
-__global__ __launch_bounds__(256) void mlstm_step_kernel(
+__global__ __launch_bounds__(1024) void mlstm_step_kernel(
     T* __restrict__ out, float* __restrict__ S, float* __restrict__ N, float* __restrict__ M,
     const T* __restrict__ proj, long ld, const float* __restrict__ gates, const float* __restrict__ b_if,
     const float* __restrict__ w, const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx,
@@ -207,7 +236,9 @@ __global__ __launch_bounds__(256) void mlstm_step_kernel(
   __shared__ float red[16];
   float* sq = sm;
   float* sk = sm + dim;
+  float* part = sm + 2 * dim;
   const int s = blockIdx.y, h = blockIdx.x, tid = threadIdx.x;
+  const int G = blockDim.x >> 8, g = tid >> 8, c0 = tid & 255;
   const long t = seq_cu[s];
   if (seq_cu[s + 1] - t <= 0) return;
   const bool carried = seq_ctx[s] - 1 > 0;
@@ -223,7 +254,7 @@ __global__ __launch_bounds__(256) void mlstm_step_kernel(
   const float m1 = fmaxf(fg + m0, ig);
   const float a = expf(fg + m0 - m1), b = expf(ig - m1);
   float nq = 0.f;
-  for (int i = tid; i < dim; i += 256) {
+  for (int i = tid; i < dim; i += blockDim.x) {
     const float q = ldf<T>(row, (long)h * dim + i) * qscale, k = ldf<T>(row, (long)(heads + h) * dim + i);
     sq[i] = q;
     sk[i] = k;
@@ -231,24 +262,44 @@ __global__ __launch_bounds__(256) void mlstm_step_kernel(
     Np[i] = nn;
     nq = __builtin_fmaf(nn, q, nq);
   }
-  nq = block_sum(nq, red);   // also the barrier after which sq / sk are read
+  nq = block_sum(nq, red);   // also the barrier after which sq / sk are read and every thread has read *mp
   if (tid == 0) *mp = m1;
   const float iden = 1.f / (fmaxf(fabsf(nq), expf(-m1)) + 1e-6f);
   const long voff = 2L * heads * dim + (long)h * vdim;
+  const int per = (dim + G - 1) / G, lo = g * per, hi = min(dim, lo + per);
   float ov[kStepCols];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < kStepCols; ++j) {
-    const int c = tid + 256 * j;
+    const int c = c0 + 256 * j;
     ov[j] = 0.f;
+    if (256 * j >= vdim) break;   // uniform over the workgroup
+    float acc = 0.f;
     if (c < vdim) {
       const float bv = b * ldf<T>(row, voff + c);
-      float acc = 0.f;
-      for (int i = 0; i < dim; ++i) {
-        const float st = __builtin_fmaf(a, carried ? Sp[(long)i * vdim + c] : 0.f, bv * sk[i]);
-        Sp[(long)i * vdim + c] = st;
-        acc = __builtin_fmaf(st, sq[i], acc);
+      float* col = Sp + c;
+      for (int i0 = lo; i0 < hi; i0 += 8) {
+        float sv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sv[u] = (carried && i0 + u < hi) ? col[(long)(i0 + u) * vdim] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (i0 + u < hi) {
+            const float st = __builtin_fmaf(a, sv[u], bv * sk[i0 + u]);
+            col[(long)(i0 + u) * vdim] = st;
+            acc = __builtin_fmaf(st, sq[i0 + u], acc);
+          }
+        }
       }
+    }
+    if (G > 1) {
+      if (g > 0) part[(g - 1) * 256 + c0] = acc;
+      __syncthreads();
+      if (g == 0)
+        for (int gg = 1; gg < G; ++gg) acc += part[(gg - 1) * 256 + c0];
+      __syncthreads();
+    }
+    if (g == 0 && c < vdim) {
       ov[j] = acc * iden;
       ss += ov[j] * ov[j];
     }
@@ -256,9 +307,10 @@ __global__ __launch_bounds__(256) void mlstm_step_kernel(
   ss = block_sum(ss, red);
   const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
   const long goff = voff + (long)heads * vdim;
+  if (g != 0) return;
 #pragma unroll
   for (int j = 0; j < kStepCols; ++j) {
-    const int c = tid + 256 * j;
+    const int c = c0 + 256 * j;
     if (c < vdim)
       stf<T>(out, (t * heads + h) * vdim + c, ov[j] * inv * w[h * vdim + c] * sigmoid_f(ldf<T>(row, goff + c)));
   }
@@ -272,20 +324,24 @@ void run(void* out, float* S, float* N, float* M, const void* proj, long ld, con
          float* scratch, int heads, int dim, int vdim, float cap, float eps, bool one_row_seqs, hipStream_t s) {
   const float qscale = 1.f / sqrtf((float)dim);
   if (one_row_seqs && vdim <= 256 * kStepCols) {
-    mlstm_step_kernel<T><<<dim3(heads, nseq), 256, 2 * dim * sizeof(float), s>>>(
+    const int G = dim >= 64 ? 4 : dim >= 16 ? 2 : 1;
+    mlstm_step_kernel<T><<<dim3(heads, nseq), 256 * G, (2 * dim + (G - 1) * 256) * sizeof(float), s>>>(
         (T*)out, S, N, M, (const T*)proj, ld, gates, b_if, norm_w, seq_cu, seq_ctx, seq_state, heads, dim, vdim, cap,
         qscale, eps);
     return;
   }
   f32x4* scr = reinterpret_cast<f32x4*>(scratch);          // [T, heads] (a, b, exp(-m), 0)
   float* o = scratch + (long)T_rows * heads * 4;             // [T, heads, vdim + 1]
+  float* vv = o + (long)T_rows * heads * (vdim + 1);         // [T, heads, vdim + 1]
+  float* qk = vv + (long)T_rows * heads * (vdim + 1);        // [T, heads, 2 dim]
+  mlstm_stage_kernel<T><<<T_rows, 256, 0, s>>>(qk, vv, (const T*)proj, ld, heads, dim, vdim, qscale);
   mlstm_gates_kernel<<<dim3(heads, nseq), 64, 0, s>>>(scr, M, gates, b_if, seq_cu, seq_ctx, seq_state, heads, cap);
   dim3 grid(heads, (vdim + 1 + kCols - 1) / kCols, nseq);
   switch (ds_of(dim)) {
 #define HS_ML(D)                                                                                                    \
   case D:                                                                                                           \
-    mlstm_scan_kernel<T, D><<<grid, kScanThreads, 0, s>>>(o, S, N, (const T*)proj, ld, scr, seq_cu, seq_ctx, seq_state, \
-                                                         heads, dim, vdim, qscale);                                 \
+    mlstm_scan_kernel<D><<<grid, kScanThreads, 0, s>>>(o, S, N, qk, vv, scr, seq_cu, seq_ctx, seq_state, heads, dim,  \
+                                                      vdim);                                                        \
     break;
     HS_ML(1) HS_ML(2) HS_ML(4) HS_ML(8) HS_ML(16)
 #undef HS_ML

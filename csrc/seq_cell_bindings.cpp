@@ -96,7 +96,7 @@ void mlstm(at::Tensor& out, at::Tensor& S, at::Tensor& N, at::Tensor& M, const a
   TORCH_CHECK(M.dim() == 2 && M.size(0) == S.size(0) && M.size(1) == heads);
   TORCH_CHECK(seq_cu.numel() == nseq + 1 && seq_state.numel() >= nseq && nseq <= 65535);
   TORCH_CHECK(!one_row_seqs || T >= nseq, "mlstm: one row per sequence");
-  TORCH_CHECK(scratch.numel() >= T * heads * (vdim + 5));
+  TORCH_CHECK(scratch.numel() >= T * heads * (2 * dim + 2 * vdim + 6));
   c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
   hipserve::launch_mlstm(out.data_ptr(), S.data_ptr<float>(), N.data_ptr<float>(), M.data_ptr<float>(), proj.data_ptr(),
                          proj.stride(0), gates.data_ptr<float>(), b_if.data_ptr<float>(), norm_w.data_ptr<float>(),

@@ -3,7 +3,9 @@ sizes that resemble a real model's layers, each beside the closest existing fami
 size: Kesirax beside a Mixtral-style model (sliding-window attention + MoE feed-forward),
 Fikizen beside a dense sliding-window model (grouped-query attention + gated dense
 feed-forward), Kemavik beside Fikizen (the other design that mixes attention layers with
-linear recurrences; its attention has no window). Random-init weights, synthetic prompts, a few layers of each (the per-layer
+linear recurrences; its attention has no window), Topezen beside Kemavik (attention layers, a
+matrix-valued recurrence and routed experts with a shared expert in both) and beside Kesirax (the
+other design with latent attention). Random-init weights, synthetic prompts, a few layers of each (the per-layer
 cost is what is compared). ``--layer-models`` picks the models; the ratios are given per pair.
 
 Per size and model, through the engine's own scheduler and step function:
@@ -94,9 +96,32 @@ def kemavik_config(name, s):
                          max_position_embeddings=16384, eos_token_id=(2,), bos_token_id=1)
 
 
+def topezen_config(name, s):
+    """Four layers: latent attention + dense PolyNorm feed-forward, matrix memory + routed experts, capped window
+    attention with kept first tokens and learned sinks + routed experts, matrix memory + dense feed-forward.
+    Matrix memory heads as in large xLSTM models: key size width / 2 and value size width over width / 256 heads."""
+    from ..config import (DenseFFSpec, HybridLayerSpec, LatentAttentionSpec, MLstmSpec, RoutedMoESpec, TopezenConfig,
+                          WindowAttentionSpec)
+
+    H, kv = s["heads"], max(1, s["heads"] // 4)
+    latent = LatentAttentionSpec(heads=H, dim=128, rot_dim=64, vdim=128, q_rank=s["width"] // 2, kv_rank=512,
+                                 scale=192 ** -0.5, rot_base=10000.0, interleaved=True, gate="channel")
+    mem = MLstmSpec(heads=s["width"] // 256, dim=128, vdim=256, gate_cap=15.0)
+    attn = WindowAttentionSpec(heads=H, kv_heads=kv, dim=128, vdim=128, scale=128 ** -0.5, window=s["window"],
+                               keep_first=64, softcap=50.0, head_norm=True, sink=True, sink_weights=True)
+    d = DenseFFSpec(s["dense_ff"], "polynorm")
+    moe = RoutedMoESpec(experts=s["experts"], top=s["top"], ff=s["ff"], shared_ff=s["ff"], groups=4, keep_groups=2,
+                        renorm=True)
+    layers = (HybridLayerSpec(latent, d), HybridLayerSpec(mem, moe), HybridLayerSpec(attn, moe), HybridLayerSpec(mem, d))
+    return TopezenConfig(name=f"topezen-{name}", hidden_size=s["width"], vocab_size=s["vocab"], layers=layers,
+                         embed_scale=float(s["width"]) ** 0.5, max_position_embeddings=16384, eos_token_id=(2,),
+                         bos_token_id=1)
+
+
 MODELS = {"kesirax": kesirax_config, "mixtral": mixtral_config, "fikizen": fikizen_config, "dense": dense_config,
-          "kemavik": kemavik_config}
-PAIRS = (("kesirax", "mixtral"), ("fikizen", "dense"), ("kemavik", "fikizen"), ("kemavik", "mixtral"))
+          "kemavik": kemavik_config, "topezen": topezen_config}
+PAIRS = (("kesirax", "mixtral"), ("fikizen", "dense"), ("kemavik", "fikizen"), ("kemavik", "mixtral"),
+         ("topezen", "kemavik"), ("topezen", "kesirax"))
 
 
 def measure(mcfg, batch, prompt_len, new_tokens, device="cuda", repeats=2):

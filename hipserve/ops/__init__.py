@@ -432,7 +432,8 @@ class KernelOps:
         return out
 
     def mlstm(self, out, state, proj, gates, b_if, norm_w, sp, eps, meta):
-        scratch = torch.empty(proj.shape[0] * sp.heads * (sp.vdim + 5), device=proj.device, dtype=torch.float32)
+        scratch = torch.empty(proj.shape[0] * sp.heads * (2 * sp.dim + 2 * sp.vdim + 6), device=proj.device,
+                              dtype=torch.float32)
         self._cell.mlstm(out, state[0], state[1], state[2], proj, gates, b_if, norm_w, meta.seq_cu, meta.seq_ctx,
                          meta.seq_state, scratch, sp.heads, sp.dim, sp.vdim, sp.gate_cap, eps, meta.max_q == 1)
 
