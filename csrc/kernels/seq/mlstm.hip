@@ -316,7 +316,7 @@ __global__ __launch_bounds__(1024) void mlstm_step_kernel(
   }
 }
 
-int ds_of(int dim) { return dim <= 16 ? 1 : dim <= 32 ? 2 : dim <= 64 ? 4 : dim <= 128 ? 8 : 16; }
+int ds_of(int dim) { return dim <= 16 ? 1 : dim <= 32 ? 2 : dim <= 64 ? 4 : dim <= 128 ? 8 : dim <= 256 ? 16 : 32; }
 
 template <typename T>
 void run(void* out, float* S, float* N, float* M, const void* proj, long ld, const float* gates, const float* b_if,
@@ -343,7 +343,7 @@ void run(void* out, float* S, float* N, float* M, const void* proj, long ld, con
     mlstm_scan_kernel<D><<<grid, kScanThreads, 0, s>>>(o, S, N, qk, vv, scr, seq_cu, seq_ctx, seq_state, heads, dim,  \
                                                       vdim);                                                        \
     break;
-    HS_ML(1) HS_ML(2) HS_ML(4) HS_ML(8) HS_ML(16)
+    HS_ML(1) HS_ML(2) HS_ML(4) HS_ML(8) HS_ML(16) HS_ML(32)
 #undef HS_ML
   }
   const long nrow = (long)T_rows * heads;
@@ -354,7 +354,7 @@ void run(void* out, float* S, float* N, float* M, const void* proj, long ld, con
 
 }  // namespace
 
-int mlstm_max_dim() { return 256; }
+int mlstm_max_dim() { return 512; }
 
 void launch_mlstm(void* out, float* S, float* N, float* M, const void* proj, long ld, const float* gates,
                   const float* b_if, const float* norm_w, const int* seq_cu, const int* seq_ctx, const int* seq_state,

@@ -115,7 +115,8 @@ def test_latent_attention_many_keys_and_what_matters(target):
 
 @pytest.mark.parametrize("target", TARGETS)
 @pytest.mark.parametrize("shape", [dict(), dict(heads=1, dim=1, vdim=1), dict(heads=5, dim=17, vdim=3, gate_cap=2.0),
-                                   dict(heads=2, dim=64, vdim=40), dict(heads=1, dim=70, vdim=130, gate_cap=30.0)])
+                                   dict(heads=2, dim=64, vdim=40), dict(heads=1, dim=70, vdim=130, gate_cap=30.0),
+                                   dict(heads=1, dim=300, vdim=20), dict(heads=1, dim=8, vdim=1100)])
 def test_matrix_memory_alone(target, shape):
     l = O.mlstm_layer(**shape)
     W = O.make_weights(O.make_config([l], width=24), seed=5)
